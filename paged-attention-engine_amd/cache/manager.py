@@ -79,17 +79,23 @@ class PagedSpec:
         return sum(t.elements_per_token() for t in self.tensors)
 
 
-def attention_pages(num_kv_heads: int, head_dim: int, window: Optional[int] = None) -> PagedSpec:
-    """Keys "k" [kv head][PAGE][head_dim] and values "v" [kv head][head_dim][PAGE] (transposed
-    within the page), as the attention kernels read them."""
+def attention_pages(num_kv_heads: int, head_dim: int, window: Optional[int] = None,
+                    value_dim: Optional[int] = None) -> PagedSpec:
+    """Keys "k" [kv head][PAGE][head_dim] and values "v" [kv head][value_dim][PAGE] (transposed
+    within the page; as wide as the keys unless `value_dim` says otherwise), as the attention kernels
+    read them."""
     return PagedSpec((PagedTensor("k", (num_kv_heads, PAGE, head_dim)),
-                      PagedTensor("v", (num_kv_heads, head_dim, PAGE))), window)
+                      PagedTensor("v", (num_kv_heads, head_dim if value_dim is None else value_dim, PAGE))), window)
 
 
 @dataclass(frozen=True)
 class StateSpec:
+    """One tensor of fixed shape that a stop keeps per request.  A stop that keeps several declares a
+    tuple of them with distinct names and finds them by name (`CacheManager.state_of`)."""
+
     shape: Tuple[int, ...]
     dtype: torch.dtype = torch.float32
+    name: str = "state"
 
 
 def bytes_of_one_page_everywhere(paged: Sequence[Optional[PagedSpec]], block_size: int, dtype: torch.dtype) -> int:
@@ -187,9 +193,15 @@ class CacheManager:
                         (len(group.entries), group.allocator.num_blocks + 1, *t.shape(block_size)),
                         dtype=dtype, device=device)
             for entry, spec in enumerate(states):
-                if spec is not None:
+                if isinstance(spec, StateSpec):
                     self.state_tensors[entry] = torch.zeros((num_slots + 1, *spec.shape), dtype=spec.dtype,
                                                             device=device)
+                elif spec is not None:
+                    names = [one.name for one in spec]
+                    if len(set(names)) != len(names):
+                        raise ValueError(f"stop {entry}: its state tensors need distinct names, got {names}")
+                    self.state_tensors[entry] = {one.name: torch.zeros((num_slots + 1, *one.shape), dtype=one.dtype,
+                                                                       device=device) for one in spec}
 
     # ------------------------------------------------------------------ lookups
     def padding_page(self, group: int) -> int:
@@ -209,8 +221,17 @@ class CacheManager:
         g, i = self._group_of_entry[entry]
         return {name: pool[i] for name, pool in self.groups[g].pools.items()}
 
-    def state_of(self, entry: int) -> torch.Tensor:
+    def state_of(self, entry: int):
+        """What stop `entry` keeps per request, [slot][*shape]: the tensor of a stop that declared one
+        `StateSpec`, a dict by name of a stop that declared several."""
         return self.state_tensors[entry]
+
+    def _state_tensors(self):
+        for held in self.state_tensors.values():
+            yield from (held.values() if isinstance(held, dict) else (held,))
+
+    def state_bytes(self) -> int:
+        return sum(t.numel() * t.element_size() for t in self._state_tensors())
 
     def storage_bytes(self) -> int:
         elem = torch.empty((), dtype=self.dtype).element_size()
@@ -235,7 +256,7 @@ class CacheManager:
         for group in self.groups:
             group.allocator.create_sequence(seq_id)
         self._tokens[seq_id] = 0
-        for tensor in self.state_tensors.values():
+        for tensor in self._state_tensors():
             tensor[slot].zero_()
         return True
 

@@ -37,13 +37,28 @@ class NormSpec(PartSpec):
 
 
 @dataclass(frozen=True)
+class FrequencyRamp:
+    """Frequencies of a rotation stretched for contexts longer than the `original` one (YaRN): a pair
+    that turns more than `fast` times over the original context keeps its frequency, one that turns
+    fewer than `slow` times has it divided by `factor`, and the pairs between are blended linearly
+    over their index; cosines and sines are multiplied by 0.1 ln(factor) + 1."""
+
+    factor: float
+    original: float
+    fast: float
+    slow: float
+
+
+@dataclass(frozen=True)
 class PositionSpec(PartSpec):
     """Rotation of query and key by absolute position; `rotary_dim` leading
-    features of each head are rotated in pairs (i, i + rotary_dim/2)."""
+    features of each head are rotated in pairs: (i, i + rotary_dim/2) for kind
+    "neox_rope", (2i, 2i + 1) for kind "interleaved_rope" (which also takes a `ramp`)."""
 
     rotary_dim: int = 0
     theta: float = 10000.0
     kind: str = "neox_rope"
+    ramp: Optional[FrequencyRamp] = None
 
 
 @dataclass(frozen=True)
@@ -63,12 +78,61 @@ class MixerSpec(PartSpec):
     window: Optional[int] = None
     position: Optional[PositionSpec] = None
     kind: str = "attention"
-    # names of the four projections below the mixer's prefix (each with ".weight" and, where the
+    # names of the four projections below the mixer's prefix (each with `weight_suffix` and, where the
     # spec says so, ".bias"): an architecture that calls them otherwise sets these, not a new mixer
     q_name: str = "q_proj"
     k_name: str = "k_proj"
     v_name: str = "v_proj"
     o_name: str = "o_proj"
+    weight_suffix: str = ".weight"
+    # what some architectures' attention has besides (None / False: not there)
+    value_dim: Optional[int] = None      # width of a value head when it differs from head_dim
+    softcap: Optional[float] = None      # scores become softcap * tanh(score / softcap)
+    sinks: bool = False                  # one learned number per query head joins the softmax's denominator
+    sink_name: str = "sinks"
+    qk_norm: Optional[str] = None        # "projection": RMS norm over the whole q and the whole k projection
+    qk_norm_eps: float = 1e-6
+    q_norm_name: str = "q_norm.weight"
+    k_norm_name: str = "k_norm.weight"
+
+    @property
+    def v_dim(self) -> int:
+        return self.head_dim if self.value_dim is None else self.value_dim
+
+    @property
+    def plain(self) -> bool:
+        """The reference's attention and nothing more: what the matrix-core kernels compute."""
+        return (self.value_dim in (None, self.head_dim) and self.softcap is None and not self.sinks
+                and self.qk_norm is None)
+
+
+@dataclass(frozen=True)
+class DeltaMixerSpec(PartSpec):
+    """The gated delta rule: a recurrent mixer with one state matrix [key_dim, value_dim] per head
+    and short causal convolutions on q, k and v.  `num_kv_heads` query/key heads of `key_dim` serve
+    `num_heads` value heads of `value_dim`."""
+
+    hidden_size: int = 0
+    num_heads: int = 0
+    num_kv_heads: int = 0
+    key_dim: int = 0
+    value_dim: int = 0
+    conv_taps: int = 4
+    norm_eps: float = 1e-6
+    unit_eps: float = 1e-6   # inside the root when q and k are made unit vectors
+    kind: str = "gated_delta"
+    q_name: str = "q"
+    k_name: str = "k"
+    v_name: str = "v"
+    gate_name: str = "g"
+    beta_name: str = "b"
+    decay_name: str = "a"
+    o_name: str = "o"
+    conv_suffix: str = ".conv"
+    a_log_name: str = "A_log"
+    dt_bias_name: str = "dt_bias"
+    norm_name: str = "norm"
+    weight_suffix: str = ""
 
 
 @dataclass(frozen=True)
@@ -81,6 +145,7 @@ class FeedForwardSpec(PartSpec):
     gate_name: str = "gate_proj"
     up_name: str = "up_proj"
     down_name: str = "down_proj"
+    weight_suffix: str = ".weight"
 
 
 @dataclass(frozen=True)
@@ -89,15 +154,16 @@ class LayerSpec:
 
     prefix: str
     mixer: PartSpec
-    feed_forward: PartSpec
+    feed_forward: Optional[PartSpec]   # None: the layer has no feed-forward (arrangements that allow it)
     mixer_norm: PartSpec
-    feed_forward_norm: PartSpec
+    feed_forward_norm: Optional[PartSpec]
     # tensor-name prefixes of the four parts below `prefix`
     mixer_prefix: str = "self_attn."
     feed_forward_prefix: str = "mlp."
     mixer_norm_prefix: str = "input_layernorm."
     feed_forward_norm_prefix: str = "post_attention_layernorm."
     arrangement: str = "prenorm"
+    residual_scale: float = 1.0  # what a branch is multiplied by before it joins the stream ("branchnorm")
 
 
 @dataclass(frozen=True)

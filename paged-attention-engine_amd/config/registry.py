@@ -29,6 +29,8 @@ def known_architectures():
 
 def read_config_dict(cfg: Mapping[str, Any]):
     archs = cfg.get("architectures")
+    if not archs and isinstance(cfg.get("architecture"), str):
+        archs = [cfg["architecture"]]  # some configurations name their one architecture in the singular
     if not archs or not isinstance(archs, (list, tuple)):
         raise ConfigError("config.json lacks the key 'architectures'")
     name = archs[0]

@@ -48,6 +48,30 @@ int pae_paged_attention_generic(int dtype, void* out, int64_t out_stride, const 
                                 const int* tok_seq, const int* block_tables, int max_blocks, int bs,
                                 int num_tokens, int nh, int nkv, int hd, float scale, int window,
                                 hipStream_t stream);
+// attention with values of their own width `vd`, a cap on the scores (0: none) and per-head sinks (null: none)
+int pae_paged_attention_capped(int dtype, void* out, int64_t out_stride, const void* q, int64_t q_stride,
+                               const void* k_cache, const void* v_cache, const int* positions, const int* tok_seq,
+                               const int* block_tables, int max_blocks, int bs, int num_tokens, int nh, int nkv, int hd,
+                               int vd, float scale, int window, float cap, const float* sinks, hipStream_t stream);
+// rows [q | k | v]: whole-projection RMS norm of q and of k (weights null: none), rotation, cache write
+int pae_qk_norm_rotate_store(int dtype, void* qkv, int64_t row_stride, int num_tokens, int nh, int nkv, int hd, int vd,
+                             const void* q_w, const void* k_w, int w_is_f32, float eps, int rot, int interleaved,
+                             const float* cos_sin, float magnitude, const int* positions, const int* tok_seq,
+                             const int* block_tables, int max_blocks, int bs, void* k_cache, void* v_cache, int write_kv,
+                             hipStream_t stream);
+// blocks that normalise a branch's output: see branch_norm.hip
+int pae_rows_from_residual(int dtype, void* out, const float* residual, int64_t n, hipStream_t stream);
+int pae_norm_scale_add(int dtype, float* residual, const void* y, int parts, int64_t part_stride, const void* weight,
+                       int w_is_f32, float eps, float scale, void* next, int num_rows, int hidden, hipStream_t stream);
+int pae_activation(int dtype, void* x, int64_t n, int kind, hipStream_t stream);
+// the gated delta rule over a step's projected rows: see delta_rule.hip
+int pae_delta_rule_step(int dtype, const void* proj, int64_t row_stride, int num_tokens, int num_seqs, const int* tok_seq,
+                        const int* positions, const int* seq_runs, const int* slots, const float* conv_w,
+                        float* conv_tail, int64_t tail_slot_stride, int taps, int G, int H, int D, int V,
+                        const float* a_log, const float* dt_bias, float unit_eps, float* state,
+                        int64_t state_slot_stride, const void* norm_w, int w_is_f32, float norm_eps, float* work,
+                        void* out, hipStream_t stream);
+int64_t pae_delta_rule_work_floats(int num_tokens, int G, int H, int D, int V);
 int pae_attn_decode_split();
 int pae_attn_decode_bf16(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* k_cache,
                          const void* v_cache, const int* dec_work, int num_dec, const int* block_tables,

@@ -13,15 +13,20 @@
 // lane = key within the chunk, with an online softmax in float32.  What a
 // (token, head) computes therefore depends on nothing but its own position:
 // not on how the step was cut, nor on what else is in the batch.
+//
+// Three things beyond the reference's attention, each switched by a parameter: values of their own
+// width `vd` (keys and queries stay `hd` wide), a cap on the scores (s <- cap * tanh(s / cap),
+// cap 0: none), and one learned sink per query head, a number that joins the softmax's denominator
+// as exp(sink) without a key or a value of its own (sinks null: none).
 #include "common.h"
 #include "api.h"
 
-template <typename T, int MAXD>  // MAXD: output features per lane, head_dim <= 64 * MAXD
+template <typename T, int MAXD>  // MAXD: output features per lane, value width <= 64 * MAXD
 __global__ void paged_attention_generic_kernel(
     T* __restrict__ out, int64_t out_stride, const T* __restrict__ q, int64_t q_stride,
     const T* __restrict__ k_cache, const T* __restrict__ v_cache, const int* __restrict__ positions,
     const int* __restrict__ tok_seq, const int* __restrict__ block_tables, int max_blocks, int bs,
-    int nh, int nkv, int hd, float scale, int window) {
+    int nh, int nkv, int hd, int vd, float scale, int window, float cap, const float* __restrict__ sinks) {
   extern __shared__ float lds[];  // [hd] query, [64] probabilities
   float* q_lds = lds;
   float* p_lds = lds + hd;
@@ -54,6 +59,7 @@ __global__ void paged_attention_generic_kernel(
       float dot = 0.f;
       for (int d = 0; d < hd; ++d) dot = fmaf(q_lds[d], to_f32(kr[d]), dot);
       s = dot * scale;
+      if (cap > 0.f) s = cap * tanhf(s / cap);
     }
     const float m_new = fmaxf(m, wave_max(s));  // finite: every chunk holds a valid key
     const float p = valid ? expf(s - m_new) : 0.f;
@@ -70,21 +76,28 @@ __global__ void paged_attention_generic_kernel(
       const float pj = p_lds[j];
       const int rj = __shfl(row, j, PAE_WAVE);
       // values are transposed within a page: [block][kv head][feature][offset in page]
-      const T* vr = v_cache + (int64_t)(rj / bs) * bs * hd + rj % bs;
+      const T* vr = v_cache + (int64_t)(rj / bs) * bs * vd + rj % bs;
 #pragma unroll
       for (int i = 0; i < MAXD; ++i) {
         const int d = lane + i * PAE_WAVE;
-        if (d < hd) acc[i] = fmaf(pj, to_f32(vr[(int64_t)d * bs]), acc[i]);
+        if (d < vd) acc[i] = fmaf(pj, to_f32(vr[(int64_t)d * bs]), acc[i]);
       }
     }
     __syncthreads();
   }
-  T* o = out + (int64_t)t * out_stride + (int64_t)head * hd;
-  const float inv = 1.0f / l;
+  T* o = out + (int64_t)t * out_stride + (int64_t)head * vd;
+  float keep = 1.f;  // what the sums keep when the sink raises the reference point
+  if (sinks) {
+    const float sink = sinks[head];
+    const float m_all = fmaxf(m, sink);
+    keep = expf(m - m_all);
+    l = l * keep + expf(sink - m_all);
+  }
+  const float inv = keep / l;
 #pragma unroll
   for (int i = 0; i < MAXD; ++i) {
     const int d = lane + i * PAE_WAVE;
-    if (d < hd) o[d] = from_f32<T>(acc[i] * inv);
+    if (d < vd) o[d] = from_f32<T>(acc[i] * inv);
   }
 }
 
@@ -92,19 +105,43 @@ template <typename T>
 static int launch_generic(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* k_cache,
                           const void* v_cache, const int* positions, const int* tok_seq,
                           const int* block_tables, int max_blocks, int bs, int num_tokens, int nh, int nkv,
-                          int hd, float scale, int window, hipStream_t stream) {
+                          int hd, int vd, float scale, int window, float cap, const float* sinks,
+                          hipStream_t stream) {
   dim3 grid(num_tokens, nh);
   const size_t lds = (size_t)(hd + PAE_WAVE) * sizeof(float);
 #define PAE_LAUNCH(MAXD)                                                                              \
   paged_attention_generic_kernel<T, MAXD><<<grid, PAE_WAVE, lds, stream>>>(                           \
       (T*)out, out_stride, (const T*)q, q_stride, (const T*)k_cache, (const T*)v_cache, positions,    \
-      tok_seq, block_tables, max_blocks, bs, nh, nkv, hd, scale, window)
-  if (hd <= 64) PAE_LAUNCH(1);
-  else if (hd <= 128) PAE_LAUNCH(2);
-  else if (hd <= 192) PAE_LAUNCH(3);
+      tok_seq, block_tables, max_blocks, bs, nh, nkv, hd, vd, scale, window, cap, sinks)
+  if (vd <= 64) PAE_LAUNCH(1);
+  else if (vd <= 128) PAE_LAUNCH(2);
+  else if (vd <= 192) PAE_LAUNCH(3);
   else PAE_LAUNCH(4);
 #undef PAE_LAUNCH
   return pae_check_launch("paged_attention_generic");
+}
+
+extern "C" int pae_paged_attention_capped(int dtype, void* out, int64_t out_stride, const void* q,
+                                          int64_t q_stride, const void* k_cache, const void* v_cache,
+                                          const int* positions, const int* tok_seq,
+                                          const int* block_tables, int max_blocks, int bs,
+                                          int num_tokens, int nh, int nkv, int hd, int vd, float scale,
+                                          int window, float cap, const float* sinks, hipStream_t stream) {
+  PAE_REQUIRE(nh > 0 && nkv > 0 && nh % nkv == 0, "attention: %d query heads over %d key/value heads", nh, nkv);
+  PAE_REQUIRE(hd > 0 && hd <= 1024, "attention: head_dim %d is outside 1..1024", hd);
+  PAE_REQUIRE(vd > 0 && vd <= 256, "attention: value width %d is outside 1..256", vd);
+  PAE_REQUIRE(bs > 0 && max_blocks > 0, "attention: bad cache geometry bs=%d max_blocks=%d", bs, max_blocks);
+  PAE_REQUIRE(window >= 0, "attention: negative window %d", window);
+  PAE_REQUIRE(cap >= 0.f, "attention: negative score cap %g", (double)cap);
+  PAE_REQUIRE(nh <= 65535, "attention: %d query heads exceed the grid", nh);
+  if (num_tokens <= 0) return 0;
+  if (dtype == PAE_F32)
+    return launch_generic<float>(out, out_stride, q, q_stride, k_cache, v_cache, positions, tok_seq, block_tables,
+                                 max_blocks, bs, num_tokens, nh, nkv, hd, vd, scale, window, cap, sinks, stream);
+  if (dtype == PAE_BF16)
+    return launch_generic<bf16_t>(out, out_stride, q, q_stride, k_cache, v_cache, positions, tok_seq, block_tables,
+                                  max_blocks, bs, num_tokens, nh, nkv, hd, vd, scale, window, cap, sinks, stream);
+  return pae_fail("attention: unknown dtype code %d", dtype);
 }
 
 extern "C" int pae_paged_attention_generic(int dtype, void* out, int64_t out_stride, const void* q,
@@ -113,17 +150,8 @@ extern "C" int pae_paged_attention_generic(int dtype, void* out, int64_t out_str
                                            const int* block_tables, int max_blocks, int bs,
                                            int num_tokens, int nh, int nkv, int hd, float scale,
                                            int window, hipStream_t stream) {
-  PAE_REQUIRE(nh > 0 && nkv > 0 && nh % nkv == 0, "attention: %d query heads over %d key/value heads", nh, nkv);
   PAE_REQUIRE(hd > 0 && hd <= 256, "attention: head_dim %d is outside 1..256", hd);
-  PAE_REQUIRE(bs > 0 && max_blocks > 0, "attention: bad cache geometry bs=%d max_blocks=%d", bs, max_blocks);
-  PAE_REQUIRE(window >= 0, "attention: negative window %d", window);
-  PAE_REQUIRE(nh <= 65535, "attention: %d query heads exceed the grid", nh);
-  if (num_tokens <= 0) return 0;
-  if (dtype == PAE_F32)
-    return launch_generic<float>(out, out_stride, q, q_stride, k_cache, v_cache, positions, tok_seq,
-                                 block_tables, max_blocks, bs, num_tokens, nh, nkv, hd, scale, window, stream);
-  if (dtype == PAE_BF16)
-    return launch_generic<bf16_t>(out, out_stride, q, q_stride, k_cache, v_cache, positions, tok_seq,
-                                  block_tables, max_blocks, bs, num_tokens, nh, nkv, hd, scale, window, stream);
-  return pae_fail("attention: unknown dtype code %d", dtype);
+  return pae_paged_attention_capped(dtype, out, out_stride, q, q_stride, k_cache, v_cache, positions, tok_seq,
+                                    block_tables, max_blocks, bs, num_tokens, nh, nkv, hd, hd, scale, window, 0.f,
+                                    nullptr, stream);
 }

@@ -1,0 +1,106 @@
+// Kernels of blocks that normalise a branch's output instead of its input, and of the plain
+// (ungated) feed-forward.
+//
+//   rows_from_residual   out[t] = T(residual[t]): the float32 stream as a product's operand
+//   norm_scale_add       residual[t] += scale * y[t] / sqrt(mean(y[t]^2) + eps) * w, and optionally
+//                        next[t] = T(residual[t]) for the product that reads the stream next
+//   activation           x <- act(x) in place: 0 gelu by erf, 1 gelu by tanh, 2 silu
+//
+// Sums, the division and the residual are float32; `y` may come as the activation type or as
+// float32 partial sums [parts][rows][hidden] of a product split along k, added here in order.
+#include "common.h"
+#include "api.h"
+
+template <typename T>
+__global__ void rows_from_residual_kernel(T* __restrict__ out, const float* __restrict__ residual, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) out[i] = from_f32<T>(residual[i]);
+}
+
+extern "C" int pae_rows_from_residual(int dtype, void* out, const float* residual, int64_t n, hipStream_t stream) {
+  if (n <= 0) return 0;
+  const unsigned blocks = (unsigned)((n + 255) / 256);
+  if (dtype == PAE_F32)
+    rows_from_residual_kernel<float><<<blocks, 256, 0, stream>>>((float*)out, residual, n);
+  else if (dtype == PAE_BF16)
+    rows_from_residual_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)out, residual, n);
+  else
+    return pae_fail("rows_from_residual: unknown dtype code %d", dtype);
+  return pae_check_launch("rows_from_residual");
+}
+
+template <typename T>
+__device__ __forceinline__ float branch_at(const void* y, int parts, int64_t part_stride, int64_t idx) {
+  if (parts == 0) return to_f32(((const T*)y)[idx]);
+  float sum = 0.f;
+  for (int p = 0; p < parts; ++p) sum += ((const float*)y)[p * part_stride + idx];
+  return sum;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void norm_scale_add_kernel(float* __restrict__ residual, const void* __restrict__ y,
+                                                             int parts, int64_t part_stride,
+                                                             const void* __restrict__ weight, int w_is_f32, float eps,
+                                                             float scale, T* __restrict__ next, int hidden) {
+  extern __shared__ float held[];  // the row of y, when it fits
+  __shared__ float scratch[4];
+  const int64_t base = (int64_t)blockIdx.x * hidden;
+  const bool keep = hidden <= 8192;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += 256) {
+    const float v = branch_at<T>(y, parts, part_stride, base + i);
+    if (keep) held[i] = v;
+    ss = fmaf(v, v, ss);
+  }
+  const float total = block_sum<4>(ss, scratch);
+  const float inv = 1.0f / sqrtf(total / (float)hidden + eps);
+  for (int i = threadIdx.x; i < hidden; i += 256) {
+    const float v = keep ? held[i] : branch_at<T>(y, parts, part_stride, base + i);
+    const float r = residual[base + i] + scale * (v * inv * load_param(weight, w_is_f32, i));
+    residual[base + i] = r;
+    if (next) next[base + i] = from_f32<T>(r);
+  }
+}
+
+extern "C" int pae_norm_scale_add(int dtype, float* residual, const void* y, int parts, int64_t part_stride,
+                                  const void* weight, int w_is_f32, float eps, float scale, void* next, int num_rows,
+                                  int hidden, hipStream_t stream) {
+  PAE_REQUIRE(parts >= 0 && num_rows >= 0 && hidden > 0, "norm_scale_add: bad sizes rows=%d H=%d parts=%d", num_rows,
+              hidden, parts);
+  if (num_rows == 0) return 0;
+  const size_t lds = hidden <= 8192 ? (size_t)hidden * sizeof(float) : 0;
+  if (dtype == PAE_F32)
+    norm_scale_add_kernel<float><<<num_rows, 256, lds, stream>>>(residual, y, parts, part_stride, weight, w_is_f32, eps,
+                                                                 scale, (float*)next, hidden);
+  else if (dtype == PAE_BF16)
+    norm_scale_add_kernel<bf16_t><<<num_rows, 256, lds, stream>>>(residual, y, parts, part_stride, weight, w_is_f32,
+                                                                  eps, scale, (bf16_t*)next, hidden);
+  else
+    return pae_fail("norm_scale_add: unknown dtype code %d", dtype);
+  return pae_check_launch("norm_scale_add");
+}
+
+__device__ __forceinline__ float act_of(float z, int kind) {
+  if (kind == 0) return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f));
+  if (kind == 1) return 0.5f * z * (1.0f + tanhf(0.79788456080286536f * (z + 0.044715f * z * z * z)));
+  return z / (1.0f + expf(-z));
+}
+
+template <typename T>
+__global__ void activation_kernel(T* __restrict__ x, int64_t n, int kind) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) x[i] = from_f32<T>(act_of(to_f32(x[i]), kind));
+}
+
+extern "C" int pae_activation(int dtype, void* x, int64_t n, int kind, hipStream_t stream) {
+  PAE_REQUIRE(kind >= 0 && kind <= 2, "activation: unknown kind %d", kind);
+  if (n <= 0) return 0;
+  const unsigned blocks = (unsigned)((n + 255) / 256);
+  if (dtype == PAE_F32)
+    activation_kernel<float><<<blocks, 256, 0, stream>>>((float*)x, n, kind);
+  else if (dtype == PAE_BF16)
+    activation_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)x, n, kind);
+  else
+    return pae_fail("activation: unknown dtype code %d", dtype);
+  return pae_check_launch("activation");
+}

@@ -67,6 +67,9 @@ class Model:
         self.embedding: Optional[torch.Tensor] = None
         self.head: Optional[Linear] = None
         self.forward_pass_count = 0
+        # for debugging a model against another implementation: called after every stop with (index,
+        # stream); the stream's residual is complete there only for blocks that leave nothing pending
+        self.residual_tap = None
 
     # ------------------------------------------------------------------ weights
     def expected_tensors(self) -> Dict[str, Tuple[int, ...]]:
@@ -155,7 +158,11 @@ class Model:
             ctx.cache_entry = index if entry.cache_from is None else entry.cache_from
             ctx.writes_cache = entry.cache_from is None
             stream.next_norm = first_norms[index + 1]
+            after = self.plan.schedule[index + 1].layer if index + 1 < len(self.plan.schedule) else None
+            stream.rows_wanted_next = after is not None and getattr(self.blocks[after], "reads_stream_rows", False)
             self.blocks[entry.layer].forward(ctx, stream)
+            if self.residual_tap is not None:
+                self.residual_tap(index, stream)
 
     # ------------------------------------------------------------------ forward
     def forward(self, ctx: StepContext, token_ids: torch.Tensor, logit_rows: torch.Tensor) -> torch.Tensor:

@@ -69,6 +69,12 @@ def _declare(lib) -> None:
         "pae_skinny_ticket_slots": [I, I],
         "pae_gemm_plain": [I, I, P, L, P, L, P, P, I, I, I, I, P],
         "pae_paged_attention_generic": [I, P, L, P, L, P, P, P, P, P, I, I, I, I, I, I, F, I, P],
+        "pae_paged_attention_capped": [I, P, L, P, L, P, P, P, P, P, I, I, I, I, I, I, I, F, I, F, P, P],
+        "pae_qk_norm_rotate_store": [I, P, L, I, I, I, I, I, P, P, I, F, I, I, P, F, P, P, P, I, I, P, P, I, P],
+        "pae_rows_from_residual": [I, P, P, L, P],
+        "pae_norm_scale_add": [I, P, P, I, L, P, I, F, F, P, I, I, P],
+        "pae_activation": [I, P, L, I, P],
+        "pae_delta_rule_step": [I, P, L, I, I, P, P, P, P, P, P, L, I, I, I, I, I, P, P, F, P, L, P, I, F, P, P, P],
         "pae_sample": [P, P, L, P, P, I, I, P, P, P, P],
         "pae_sample_chunks": [I],
         "pae_sample_static": [P, P, L, P, P, I, I, P],
@@ -95,6 +101,8 @@ def _declare(lib) -> None:
         fn.restype = c_int
     lib.pae_skinny_ticket_floats.argtypes = [I, I, I]
     lib.pae_skinny_ticket_floats.restype = c_int64
+    lib.pae_delta_rule_work_floats.argtypes = [I, I, I, I, I]
+    lib.pae_delta_rule_work_floats.restype = c_int64
 
 
 def _check(code: int) -> None:
@@ -860,6 +868,161 @@ def paged_attention_generic(out: torch.Tensor, q: torch.Tensor, k_cache: torch.T
         code_of(q.dtype), out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0), k_cache.data_ptr(),
         v_cache.data_ptr(), positions.data_ptr(), tok_seq.data_ptr(), block_tables.data_ptr(),
         block_tables.shape[1], bs, T, nh, nkv, hd, float(scale), int(window), _stream()))
+
+
+def _check_pools_wide(k_cache, v_cache, nkv: int, bs: int, hd: int, vd: int) -> None:
+    """Keys [block][kv head][bs][hd]; values of width vd transposed within the page, [block][kv head][vd][bs]."""
+    assert tuple(k_cache.shape[1:]) == (nkv, bs, hd) and k_cache.is_contiguous()
+    assert tuple(v_cache.shape) == (k_cache.shape[0], nkv, vd, bs) and v_cache.is_contiguous()
+    assert k_cache.dtype == v_cache.dtype
+
+
+def paged_attention_capped(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                           positions: torch.Tensor, tok_seq: torch.Tensor, block_tables: torch.Tensor,
+                           nh: int, nkv: int, hd: int, vd: int, scale: float, window: int, softcap: float = 0.0,
+                           sinks: Optional[torch.Tensor] = None) -> None:
+    """`paged_attention_generic` with values of width `vd` (out[t, h*vd:(h+1)*vd]), scores capped by
+    softcap * tanh(s / softcap) (0: no cap) and one sink per query head in the softmax's denominator
+    (`sinks` float32 [nh], None: no sinks)."""
+    _not_while_recording("paged_attention_capped")
+    _gpu(out, q, k_cache, v_cache, positions, tok_seq, block_tables, sinks)
+    T = q.shape[0]
+    bs = k_cache.shape[2]
+    assert q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= nh * hd and q.dtype == k_cache.dtype == out.dtype
+    assert out.shape[0] == T and out.stride(1) == 1 and out.shape[1] >= nh * vd
+    _check_pools_wide(k_cache, v_cache, nkv, bs, hd, vd)
+    assert positions.dtype == torch.int32 and positions.numel() == T
+    assert tok_seq.dtype == torch.int32 and tok_seq.numel() == T
+    assert block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous()
+    if sinks is not None:
+        assert sinks.dtype == torch.float32 and sinks.numel() == nh and sinks.is_contiguous()
+    _check(library().pae_paged_attention_capped(
+        code_of(q.dtype), out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0), k_cache.data_ptr(),
+        v_cache.data_ptr(), positions.data_ptr(), tok_seq.data_ptr(), block_tables.data_ptr(),
+        block_tables.shape[1], bs, T, nh, nkv, hd, vd, float(scale), int(window), float(softcap), _ptr(sinks),
+        _stream()))
+
+
+def qk_norm_rotate_store(qkv: torch.Tensor, nh: int, nkv: int, hd: int, vd: int, q_weight: Optional[torch.Tensor],
+                         k_weight: Optional[torch.Tensor], eps: float, rot: int, interleaved: bool,
+                         cos_sin: Optional[torch.Tensor], magnitude: float, positions: torch.Tensor,
+                         tok_seq: Optional[torch.Tensor], block_tables: Optional[torch.Tensor], block_size: int,
+                         k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor]) -> None:
+    """Rows [q: nh x hd | k: nkv x hd | v: nkv x vd]: with weights, q and k are each divided by the root
+    mean square of their whole projection and multiplied by the weight; the first `rot` features of
+    every q and k head are rotated by `cos_sin` times `magnitude` (pairs (2i, 2i+1) if `interleaved`,
+    else (i, i + rot/2)); queries are written back in place, keys and values to their cache slots
+    (`k_cache` None: nkv must be 0 and nothing is stored)."""
+    _not_while_recording("qk_norm_rotate_store")
+    _gpu(qkv, q_weight, k_weight, cos_sin, positions, tok_seq, block_tables, k_cache, v_cache)
+    T = qkv.shape[0]
+    assert qkv.dim() == 2 and qkv.stride(1) == 1 and positions.dtype == torch.int32 and positions.numel() == T
+    write = k_cache is not None
+    assert write or nkv == 0
+    _check_cos_sin(cos_sin, rot, T)
+    wf = 0
+    if q_weight is not None:
+        assert q_weight.numel() == nh * hd and q_weight.is_contiguous()
+        assert nkv == 0 or (k_weight is not None and k_weight.numel() == nkv * hd and k_weight.dtype == q_weight.dtype)
+        wf = _param(q_weight)[1]
+    max_blocks = 0
+    if write:
+        assert k_cache.dtype == qkv.dtype == v_cache.dtype
+        assert tok_seq.dtype == torch.int32 and tok_seq.numel() == T
+        assert block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous()
+        _check_pools_wide(k_cache, v_cache, nkv, block_size, hd, vd)
+        max_blocks = block_tables.shape[1]
+    _check(library().pae_qk_norm_rotate_store(
+        code_of(qkv.dtype), qkv.data_ptr(), qkv.stride(0), T, nh, nkv, hd, vd, _ptr(q_weight), _ptr(k_weight), wf,
+        float(eps), rot, 1 if interleaved else 0, _ptr(cos_sin) if rot else None, float(magnitude),
+        positions.data_ptr(), _ptr(tok_seq), _ptr(block_tables), max_blocks, block_size, _ptr(k_cache), _ptr(v_cache),
+        1 if write else 0, _stream()))
+
+
+def rows_from_residual(residual: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """The float32 stream [T, H] as rows of `dtype` for a matrix product (float32: the stream itself)."""
+    _not_while_recording("rows_from_residual")
+    _gpu(residual)
+    assert residual.dtype == torch.float32 and residual.is_contiguous()
+    if dtype == torch.float32:
+        return residual
+    out = torch.empty(residual.shape, dtype=dtype, device=residual.device)
+    _check(library().pae_rows_from_residual(code_of(dtype), out.data_ptr(), residual.data_ptr(), residual.numel(),
+                                            _stream()))
+    return out
+
+
+def norm_scale_add(residual: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: float, scale: float,
+                   next_rows: Optional[torch.Tensor] = None) -> None:
+    """residual[t] += scale * y[t] / sqrt(mean(y[t]^2) + eps) * weight.  `y`: [T, H] in the activation
+    type, or float32 partial sums [P, T, H] added in order.  `next_rows` [T, H] (the type of the
+    activations) receives the new residual rounded to it."""
+    _not_while_recording("norm_scale_add")
+    _gpu(residual, y, weight, next_rows)
+    T, H = residual.shape
+    assert residual.dtype == torch.float32 and residual.is_contiguous() and y.is_contiguous()
+    parts, stride = 0, 0
+    if y.dim() == 3:
+        assert y.dtype == torch.float32 and tuple(y.shape[1:]) == (T, H)
+        parts, stride = y.shape[0], T * H
+        dtype = next_rows.dtype if next_rows is not None else torch.bfloat16
+    else:
+        assert tuple(y.shape) == (T, H)
+        dtype = y.dtype
+    if next_rows is not None:
+        assert tuple(next_rows.shape) == (T, H) and next_rows.is_contiguous() and next_rows.dtype == dtype
+    assert weight.numel() == H
+    wp, wf = _param(weight)
+    _check(library().pae_norm_scale_add(code_of(dtype), residual.data_ptr(), y.data_ptr(), parts, stride, wp, wf,
+                                        float(eps), float(scale), _ptr(next_rows), T, H, _stream()))
+
+
+ACTIVATIONS = {"gelu": 0, "gelu_tanh": 1, "silu": 2}
+
+
+def activation(x: torch.Tensor, kind: str) -> None:
+    """x <- act(x) in place, computed in float32: "gelu" (by erf), "gelu_tanh", "silu"."""
+    _not_while_recording("activation")
+    _gpu(x)
+    assert x.is_contiguous() and kind in ACTIVATIONS
+    _check(library().pae_activation(code_of(x.dtype), x.data_ptr(), x.numel(), ACTIVATIONS[kind], _stream()))
+
+
+def delta_rule_step(proj: torch.Tensor, out: torch.Tensor, tok_seq: torch.Tensor, positions: torch.Tensor,
+                    seq_runs: torch.Tensor, slots: torch.Tensor, conv_w: torch.Tensor, conv_tail: torch.Tensor,
+                    state: torch.Tensor, a_log: torch.Tensor, dt_bias: torch.Tensor, norm_w: torch.Tensor,
+                    G: int, H: int, D: int, V: int, taps: int, unit_eps: float, norm_eps: float) -> None:
+    """The gated delta rule over a step's rows.  `proj` [T, 2GD + 2HV + 2H] holds per token
+    [q | k | v | gate | b | a]; `seq_runs` int32 [S, 4] = (first row, rows, tokens before, 0) per
+    sequence; `slots` int32 [S]; `conv_w` float32 [2GD + HV, taps]; `conv_tail` float32
+    [slots, taps - 1, 2GD + HV] and `state` float32 [slots, H, V, D] are the requests' state, read
+    and moved on; `out` [T, H * V] receives the normed, gated read-out in proj's type."""
+    _not_while_recording("delta_rule_step")
+    _gpu(proj, out, tok_seq, positions, seq_runs, slots, conv_w, conv_tail, state, a_log, dt_bias, norm_w)
+    T, S = proj.shape[0], seq_runs.shape[0]
+    C = 2 * G * D + H * V
+    assert proj.dim() == 2 and proj.stride(1) == 1 and proj.shape[1] == C + H * V + 2 * H
+    assert out.shape == (T, H * V) and out.is_contiguous() and out.dtype == proj.dtype
+    for t, n in ((tok_seq, T), (positions, T), (slots, S)):
+        assert t.dtype == torch.int32 and t.numel() >= n and t.is_contiguous()
+    assert seq_runs.dtype == torch.int32 and seq_runs.shape == (S, 4) and seq_runs.is_contiguous()
+    assert seq_runs.data_ptr() % 16 == 0
+    assert conv_w.dtype == torch.float32 and conv_w.shape == (C, taps) and conv_w.is_contiguous()
+    assert conv_tail.dtype == torch.float32 and tuple(conv_tail.shape[1:]) == (max(taps - 1, 0), C)
+    assert conv_tail.stride(2) == 1 and (taps == 1 or conv_tail.stride(1) == C)
+    assert state.dtype == torch.float32 and tuple(state.shape[1:]) == (H, V, D) and state[0].is_contiguous()
+    assert state.shape[0] == conv_tail.shape[0]
+    for t in (a_log, dt_bias):
+        assert t.dtype == torch.float32 and t.numel() == H and t.is_contiguous()
+    assert norm_w.numel() == V
+    wp, wf = _param(norm_w)
+    lib = library()
+    work = torch.empty(lib.pae_delta_rule_work_floats(T, G, H, D, V), dtype=torch.float32, device=proj.device)
+    _check(lib.pae_delta_rule_step(
+        code_of(proj.dtype), proj.data_ptr(), proj.stride(0), T, S, tok_seq.data_ptr(), positions.data_ptr(),
+        seq_runs.data_ptr(), slots.data_ptr(), conv_w.data_ptr(), conv_tail.data_ptr(), conv_tail.stride(0), taps, G, H,
+        D, V, a_log.data_ptr(), dt_bias.data_ptr(), float(unit_eps), state.data_ptr(), state.stride(0), wp, wf,
+        float(norm_eps), work.data_ptr(), out.data_ptr(), _stream()))
 
 
 def mfma_attention_supported(dtype: torch.dtype, nh: int, nkv: int, hd: int, bs: int) -> bool:

@@ -16,6 +16,14 @@ rotation + store for up to 64 rows, rotation + store above).
 
 A stop that borrows another stop's cache projects queries only and reads keys
 and values written by the owner.
+
+Beyond the reference's attention, each switched by the spec and absent when it says nothing:
+values of a width of their own (`value_dim`), an RMS norm of the whole query projection and of the
+whole key projection before the rotation (`qk_norm = "projection"`), scores capped by
+softcap * tanh(score / softcap), and a learned sink per query head that joins the softmax's
+denominator as exp(sink) without a key or a value (`sinks`).  A spec with any of them takes the
+path `_forward_wide`: the projection, then one kernel that norms, rotates and stores, then the
+attention kernel that knows caps, sinks and value widths.
 """
 
 from __future__ import annotations
@@ -24,7 +32,7 @@ import torch
 
 from ..cache.manager import attention_pages
 from ..kernels import lib as K
-from .base import POSITION_ENCODINGS, OwedRows, Part, StepShape, build_part, plain_rows, register_mixer
+from .base import POSITION_ENCODINGS, OwedRows, Part, ScaleShape, StepShape, build_part, plain_rows, register_mixer
 from .linear import Linear, rows_a_graph_may_hold
 
 WORK_LISTS = ("paged attention work lists", K.PREFILL_TILE)
@@ -56,8 +64,14 @@ class PagedAttention(Part):
         super().__init__(spec, dtype, device)
         if spec.num_heads % spec.num_kv_heads:
             raise ValueError(f"{spec.num_heads} query heads over {spec.num_kv_heads} key/value heads")
-        if spec.head_dim % 16 or not 16 <= spec.head_dim <= 256:
+        if spec.plain and (spec.head_dim % 16 or not 16 <= spec.head_dim <= 256):
             raise ValueError(f"head_dim {spec.head_dim}: the attention kernels take multiples of 16 up to 256")
+        if not spec.plain and not (0 < spec.head_dim <= 1024 and 0 < spec.v_dim <= 256):
+            raise ValueError(f"head_dim {spec.head_dim} / value_dim {spec.v_dim}: the attention kernel takes up to 1024 / 256")
+        if spec.qk_norm not in (None, "projection"):
+            raise ValueError(f"qk_norm '{spec.qk_norm}' is not known (known: projection)")
+        if not spec.plain and (spec.qkv_bias or spec.out_bias):
+            raise ValueError("an attention with value widths, caps, sinks or query/key norms takes no biases")
         self.position = (build_part(POSITION_ENCODINGS, "position encoding", spec.position, dtype, device)
                          if spec.position is not None else
                          POSITION_ENCODINGS["none"](None, dtype, device))
@@ -75,7 +89,7 @@ class PagedAttention(Part):
         product are all this mixer launches (a rotation that hands out its table runs inside the first)."""
         s = self.spec
         group = s.num_heads // s.num_kv_heads
-        return (self.dtype == torch.bfloat16 and 0 < rows <= K.program_max_rows() and self._matrix_cores(block_size)
+        return (s.plain and self.dtype == torch.bfloat16 and 0 < rows <= K.program_max_rows() and self._matrix_cores(block_size)
                 and s.head_dim in (64, 128) and group * s.head_dim <= 1024 and not s.out_bias
                 and hasattr(self.position, "rotary_table") and s.hidden_size % 8 == 0
                 and getattr(s.position, "rotary_dim", 0) % 16 == 0
@@ -85,24 +99,29 @@ class PagedAttention(Part):
                     s.hidden_size, s.num_heads * s.head_dim, rows)))
 
     def paged_spec(self):
-        return attention_pages(self.spec.num_kv_heads, self.spec.head_dim, self.spec.window)
+        return attention_pages(self.spec.num_kv_heads, self.spec.head_dim, self.spec.window, self.spec.value_dim)
 
     def _matrix_cores(self, block_size: int) -> bool:
         s = self.spec
         return K.mfma_attention_supported(self.dtype, s.num_heads, s.num_kv_heads, s.head_dim, block_size)
 
     def step_lists_key(self, block_size: int):
-        return WORK_LISTS if self._matrix_cores(block_size) else None
+        return WORK_LISTS if self.spec.plain and self._matrix_cores(block_size) else None
 
     def step_lists(self, shape: StepShape):
         return attention_work_lists(shape)
 
     def tensors(self, prefix):
         s = self.spec
-        out = {prefix + s.q_name + ".weight": (s.num_heads * s.head_dim, s.hidden_size),
-               prefix + s.k_name + ".weight": (s.num_kv_heads * s.head_dim, s.hidden_size),
-               prefix + s.v_name + ".weight": (s.num_kv_heads * s.head_dim, s.hidden_size),
-               prefix + s.o_name + ".weight": (s.hidden_size, s.num_heads * s.head_dim)}
+        out = {prefix + s.q_name + s.weight_suffix: (s.num_heads * s.head_dim, s.hidden_size),
+               prefix + s.k_name + s.weight_suffix: (s.num_kv_heads * s.head_dim, s.hidden_size),
+               prefix + s.v_name + s.weight_suffix: (s.num_kv_heads * s.v_dim, s.hidden_size),
+               prefix + s.o_name + s.weight_suffix: (s.hidden_size, s.num_heads * s.v_dim)}
+        if s.qk_norm:
+            out[prefix + s.q_norm_name] = ScaleShape((s.num_heads * s.head_dim,))
+            out[prefix + s.k_norm_name] = ScaleShape((s.num_kv_heads * s.head_dim,))
+        if s.sinks:
+            out[prefix + s.sink_name] = (s.num_heads,)
         if s.qkv_bias:
             out[prefix + s.q_name + ".bias"] = (s.num_heads * s.head_dim,)
             out[prefix + s.k_name + ".bias"] = (s.num_kv_heads * s.head_dim,)
@@ -114,13 +133,19 @@ class PagedAttention(Part):
     def bind(self, prefix, weights):
         s = self.spec
         names = (s.q_name, s.k_name, s.v_name)
-        w = torch.cat([weights[prefix + n + ".weight"] for n in names], dim=0)
+        w = torch.cat([weights[prefix + n + s.weight_suffix] for n in names], dim=0)
         b = (torch.cat([weights[prefix + n + ".bias"] for n in names], dim=0) if s.qkv_bias else None)
         self.qkv = Linear(self.matrix(w), None if b is None else self.vector(b))
         nq = s.num_heads * s.head_dim
         self.q_only = Linear(self.qkv.weight[:nq], None if b is None else self.qkv.bias[:nq])
         ob = weights[prefix + s.o_name + ".bias"] if s.out_bias else None
-        self.out = Linear(self.matrix(weights[prefix + s.o_name + ".weight"]), None if ob is None else self.vector(ob))
+        self.out = Linear(self.matrix(weights[prefix + s.o_name + s.weight_suffix]), None if ob is None else self.vector(ob))
+        self.q_norm = self.k_norm = self.sinks = None
+        if s.qk_norm:
+            self.q_norm = self.vector(weights[prefix + s.q_norm_name])
+            self.k_norm = self.vector(weights[prefix + s.k_norm_name])
+        if s.sinks:  # sinks enter the softmax, which is float32
+            self.sinks = weights[prefix + s.sink_name].to(device=self.device, dtype=torch.float32).contiguous()
 
     def _project_encode_store(self, ctx, x, k_cache, v_cache, table):
         """Queries (and, at a stop that owns its cache, keys and values) of the step's tokens:
@@ -162,9 +187,35 @@ class PagedAttention(Part):
                         k_cache, v_cache, bias)
         return qkv
 
+    def _forward_wide(self, ctx, x):
+        """The path of a spec that is not `plain`: see the module's text."""
+        s = self.spec
+        pages = ctx.cache.pages_of(ctx.cache_entry)
+        table = ctx.block_tables[ctx.cache.group_of(ctx.cache_entry)]
+        if ctx.writes_cache:
+            qkv, nkv, k_cache, v_cache = self.qkv(x), s.num_kv_heads, pages["k"], pages["v"]
+        else:
+            qkv, nkv, k_cache, v_cache = self.q_only(x), 0, None, None
+        rotary = getattr(self.position, "rotary_table", None)
+        if rotary is None and s.position is not None:
+            raise ValueError("an attention with value widths, caps, sinks or query/key norms rotates by a table")
+        rot, cos_sin = rotary(ctx) if rotary is not None else (0, None)
+        K.qk_norm_rotate_store(qkv, s.num_heads, nkv, s.head_dim, s.v_dim, self.q_norm, self.k_norm if nkv else None,
+                               s.qk_norm_eps, rot, bool(getattr(self.position, "interleaved", False)), cos_sin,
+                               float(getattr(self.position, "magnitude", 1.0)), ctx.positions,
+                               ctx.tok_seq if nkv else None, table if nkv else None, ctx.cache.block_size,
+                               k_cache, v_cache)
+        attn = torch.empty((qkv.shape[0], s.num_heads * s.v_dim), dtype=qkv.dtype, device=qkv.device)
+        K.paged_attention_capped(attn, qkv, pages["k"], pages["v"], ctx.positions, ctx.tok_seq, table, s.num_heads,
+                                 s.num_kv_heads, s.head_dim, s.v_dim, s.scale, s.window or 0, s.softcap or 0.0,
+                                 self.sinks)
+        return self.out.branch(attn, ctx.sink)
+
     def forward(self, ctx, x):
         """`x`: normalised activations, or `OwedRows` (the projection then pays their scale)."""
         s = self.spec
+        if not s.plain:
+            return self._forward_wide(ctx, plain_rows(x))
         pages = ctx.cache.pages_of(ctx.cache_entry)  # as declared in `paged_spec`
         k_cache, v_cache = pages["k"], pages["v"]
         table = ctx.block_tables[ctx.cache.group_of(ctx.cache_entry)]

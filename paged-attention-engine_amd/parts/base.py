@@ -83,6 +83,11 @@ class ResidualStream:
         self.owed: Optional[OwedRows] = None
         self.owed_to: Optional[object] = None
         self.next_norm: Optional[object] = None  # set by the model: the norm that reads the stream after this block
+        # for blocks whose branches read the stream itself: the residual rounded to the activation type,
+        # left by the kernel that last wrote it (None: nobody has), and whether the block after this one
+        # is such a block and will want them (set by the model)
+        self.rows: Optional[torch.Tensor] = None
+        self.rows_wanted_next = False
 
 
 class BranchSink:

@@ -73,6 +73,89 @@ class PreNormBlock:
         ctx.sink = None
 
 
+@register_block("branchnorm")
+class BranchNormBlock:
+    """The norm on each branch's output, and the branches read the stream itself:
+    x <- x + m * norm1(mixer(x)); x <- x + m * norm2(feed_forward(x)), m = `residual_scale`.
+    A layer whose spec names no feed-forward has the first half only.  The stream is float32; a
+    branch's product reads it rounded to the activation type, which the kernel that adds a branch
+    writes on the way for the branch after it (`stream.rows`)."""
+
+    reads_stream_rows = True
+
+    def __init__(self, layer_spec, dtype, device):
+        self.spec = layer_spec
+        self.dtype = dtype
+        self.mixer = build_part(MIXERS, "mixer", layer_spec.mixer, dtype, device)
+        self.mixer_out_norm = build_part(NORMS, "norm", layer_spec.mixer_norm, dtype, device)
+        self.feed_forward = self.feed_forward_out_norm = None
+        if layer_spec.feed_forward is not None:
+            self.feed_forward = build_part(FEED_FORWARDS, "feed-forward", layer_spec.feed_forward, dtype, device)
+            self.feed_forward_out_norm = build_part(NORMS, "norm", layer_spec.feed_forward_norm, dtype, device)
+        for norm in (self.mixer_out_norm, self.feed_forward_out_norm):
+            if norm is not None and not hasattr(norm, "add_scaled"):
+                raise ValueError(f"the norm '{norm.spec.kind}' cannot stand on a branch's output (no add_scaled)")
+
+    def _named(self):
+        s = self.spec
+        out = [(self.mixer_out_norm, s.prefix + s.mixer_norm_prefix), (self.mixer, s.prefix + s.mixer_prefix)]
+        if self.feed_forward is not None:
+            out += [(self.feed_forward_out_norm, s.prefix + s.feed_forward_norm_prefix),
+                    (self.feed_forward, s.prefix + s.feed_forward_prefix)]
+        return out
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(part.graph_safe for part, _ in self._named())
+
+    @property
+    def graph_max_rows(self):
+        limits = [part.graph_max_rows for part, _ in self._named() if part.graph_max_rows is not None]
+        return min(limits) if limits else None
+
+    def parts(self):
+        return [part for part, _ in self._named()]
+
+    def tensors(self):
+        out = {}
+        for part, prefix in self._named():
+            out.update(part.tensors(prefix))
+        return out
+
+    def bind(self, weights):
+        for part, prefix in self._named():
+            part.bind(prefix, weights)
+
+    def _rows(self, stream: ResidualStream):
+        """The stream as a product's operand: what the branch before left, or a cast of the residual."""
+        from ..kernels import lib as K
+        rows = getattr(stream, "rows", None)
+        stream.rows = None
+        return rows if rows is not None else K.rows_from_residual(stream.residual, self.dtype)
+
+    def _join(self, stream: ResidualStream, norm, y, more_follows: bool) -> None:
+        import torch
+        nxt = None
+        if more_follows and self.dtype != torch.float32:
+            nxt = torch.empty(stream.residual.shape, dtype=self.dtype, device=stream.residual.device)
+        norm.add_scaled(stream.residual, y, self.spec.residual_scale, nxt)
+        stream.rows = nxt
+
+    def forward(self, ctx, stream: ResidualStream) -> None:
+        if stream.pending is not None or stream.owed is not None:
+            raise ValueError("a block with its norms on the branches' outputs follows one that left a branch pending")
+        ctx.sink = None
+        has_ff = self.feed_forward is not None
+        y = self.mixer.forward(ctx, self._rows(stream))
+        # the rows of the new stream are wanted by this block's feed-forward, or by a block of this
+        # kind that follows (the model says whether one does)
+        follows = bool(getattr(stream, "rows_wanted_next", False))
+        self._join(stream, self.mixer_out_norm, y, has_ff or follows)
+        if has_ff:
+            y = self.feed_forward.forward(ctx, self._rows(stream))
+            self._join(stream, self.feed_forward_out_norm, y, follows)
+
+
 def build_block(layer_spec, dtype, device):
     if layer_spec.arrangement not in BLOCKS:
         raise KeyError(f"no block arrangement '{layer_spec.arrangement}'; known: {', '.join(sorted(BLOCKS))}")

@@ -1,6 +1,7 @@
-"""Dense gated feed-forward: down(silu(gate(x)) * up(x)), no biases
+"""Feed-forwards.  "swiglu", the dense gated one: down(silu(gate(x)) * up(x)), no biases
 (engine/model.py:317-320 of the reference).  gate and up are one product over
-concatenated weights; the gate is applied in float32 and rounded once."""
+concatenated weights; the gate is applied in float32 and rounded once.  "dense", the plain
+one: down(act(up(x))), act one of `kernels.lib.ACTIVATIONS`, applied in float32."""
 
 from __future__ import annotations
 
@@ -26,15 +27,15 @@ class SwiGLU(Part):
 
     def tensors(self, prefix):
         s = self.spec
-        return {prefix + s.gate_name + ".weight": (s.intermediate_size, s.hidden_size),
-                prefix + s.up_name + ".weight": (s.intermediate_size, s.hidden_size),
-                prefix + s.down_name + ".weight": (s.hidden_size, s.intermediate_size)}
+        return {prefix + s.gate_name + s.weight_suffix: (s.intermediate_size, s.hidden_size),
+                prefix + s.up_name + s.weight_suffix: (s.intermediate_size, s.hidden_size),
+                prefix + s.down_name + s.weight_suffix: (s.hidden_size, s.intermediate_size)}
 
     BLOCK = 8  # gate and up rows alternate in blocks of this many (the skinny product's gated epilogue)
 
     def bind(self, prefix, weights):
         s = self.spec
-        gate, up = weights[prefix + s.gate_name + ".weight"], weights[prefix + s.up_name + ".weight"]
+        gate, up = weights[prefix + s.gate_name + s.weight_suffix], weights[prefix + s.up_name + s.weight_suffix]
         inter, hidden = gate.shape
         self.block = self.BLOCK if (self.dtype == torch.bfloat16 and inter % self.BLOCK == 0) else 0
         if self.block:
@@ -44,7 +45,7 @@ class SwiGLU(Part):
         else:
             gate_up = torch.cat([gate, up], dim=0)
         self.gate_up = Linear(self.matrix(gate_up))
-        self.down = Linear(self.matrix(weights[prefix + s.down_name + ".weight"]))
+        self.down = Linear(self.matrix(weights[prefix + s.down_name + s.weight_suffix]))
 
     def decode_fusable(self, rows: int, block_size: int) -> bool:
         s = self.spec
@@ -65,4 +66,36 @@ class SwiGLU(Part):
                           row_scale=x.row_scale if isinstance(x, OwedRows) else None)
         else:
             K.swiglu(act, self.gate_up(plain_rows(x)), self.block)
+        return self.down.branch(act, getattr(ctx, "sink", None))
+
+
+@register_feed_forward("dense")
+class DenseFeedForward(Part):
+    """down(act(up(x))), no gate, no biases.  `spec.activation`: "gelu" (the exact one, by erf),
+    "gelu_tanh" or "silu"."""
+
+    graph_safe = True
+
+    def __init__(self, spec, dtype, device):
+        super().__init__(spec, dtype, device)
+        if spec.activation not in K.ACTIVATIONS:
+            raise ValueError(f"activation '{spec.activation}' is not one of {', '.join(K.ACTIVATIONS)}")
+
+    @property
+    def graph_max_rows(self):
+        return rows_a_graph_may_hold(self.dtype, self.spec.hidden_size, self.spec.intermediate_size)
+
+    def tensors(self, prefix):
+        s = self.spec
+        return {prefix + s.up_name + s.weight_suffix: (s.intermediate_size, s.hidden_size),
+                prefix + s.down_name + s.weight_suffix: (s.hidden_size, s.intermediate_size)}
+
+    def bind(self, prefix, weights):
+        s = self.spec
+        self.up = Linear(self.matrix(weights[prefix + s.up_name + s.weight_suffix]))
+        self.down = Linear(self.matrix(weights[prefix + s.down_name + s.weight_suffix]))
+
+    def forward(self, ctx, x):
+        act = self.up(plain_rows(x))
+        K.activation(act, self.spec.activation)
         return self.down.branch(act, getattr(ctx, "sink", None))

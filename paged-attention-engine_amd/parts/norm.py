@@ -56,3 +56,10 @@ class RMSNorm(Part):
         if rows is None:
             stream.pending = None
         return out
+
+    def add_scaled(self, residual: torch.Tensor, y: torch.Tensor, scale: float,
+                   next_rows: Optional[torch.Tensor] = None) -> None:
+        """The norm on a branch's output: residual += scale * norm(y), in float32 (`y` in the activation
+        type, or float32 partial sums [P, T, H]); `next_rows` receives the new residual in the
+        activation type, for the product that reads the stream next."""
+        K.norm_scale_add(residual, y, self.weight, self.spec.eps, scale, next_rows)

@@ -15,6 +15,8 @@ mixer run the rotation inside its own fused kernels.
 
 from __future__ import annotations
 
+import math
+
 import torch
 
 from ..kernels import lib as K
@@ -50,6 +52,61 @@ class NeoxRope(Part):
         rot, table = self.rotary_table(ctx)
         if rot:
             K.rotate_heads(x, num_heads, head_dim, rot, table, ctx.positions)
+
+
+def ramped_frequencies(rot: int, theta: float, ramp) -> "tuple[torch.Tensor, float]":
+    """(float32 frequency of every pair, multiplier of cosines and sines) of a rotation whose
+    frequencies are stretched by `ramp` (a `FrequencyRamp`, or None for the plain theta ** (-2i / rot)).
+    With turns(i) = original * f_i / (2 pi), the number of turns pair i makes over the original context:
+    the index at which a pair makes t turns is rot * ln(original / (2 pi t)) / (2 ln theta); pairs up to
+    the index of `fast` turns keep f_i, pairs from the index of `slow` turns on get f_i / factor, and
+    the pairs between blend the two linearly in the index.  Formed in float64, rounded once."""
+    i = torch.arange(rot // 2, dtype=torch.float64)
+    freq = theta ** (-2.0 * i / rot)
+    if ramp is None:
+        return freq.to(torch.float32), 1.0
+
+    def index_of(turns: float) -> float:
+        return rot * math.log(ramp.original / (2.0 * math.pi * turns)) / (2.0 * math.log(theta))
+
+    low = max(math.floor(index_of(ramp.fast)), 0)
+    high = min(math.ceil(index_of(ramp.slow)), rot - 1)
+    blend = torch.clamp((i - low) / max(high - low, 0.001), 0.0, 1.0)
+    freq = freq / ramp.factor * blend + freq * (1.0 - blend)
+    return freq.to(torch.float32), 0.1 * math.log(ramp.factor) + 1.0
+
+
+@register_position_encoding("interleaved_rope")
+class InterleavedRope(Part):
+    """Rotation of the pairs (2i, 2i + 1) of each head's first `rotary_dim` features by
+    position * f_i, with optionally stretched frequencies (`spec.ramp`) and cosines and sines
+    multiplied by `magnitude`.  Angles are float32 products of the position and the float32 frequency."""
+
+    graph_safe = True
+    interleaved = True
+
+    def __init__(self, spec, dtype, device):
+        super().__init__(spec, dtype, device)
+        if spec.rotary_dim % 2:
+            raise ValueError(f"rotary_dim {spec.rotary_dim} must be even")
+        freq, self.magnitude = ramped_frequencies(spec.rotary_dim, spec.theta, spec.ramp)
+        self.inv_freq = freq.to(device)
+
+    def rotary_table(self, ctx):
+        rot = self.spec.rotary_dim
+        if not rot:
+            return 0, None
+        key = ("interleaved_rope", rot, self.spec.theta, self.spec.ramp)
+        table = ctx.memo.get(key)
+        if table is None:
+            table = ctx.memo[key] = K.rope_table(ctx.positions, self.inv_freq)
+        return rot, table
+
+    def encode(self, ctx, x: torch.Tensor, num_heads: int, head_dim: int) -> None:
+        rot, table = self.rotary_table(ctx)
+        if rot:
+            K.qk_norm_rotate_store(x, num_heads, 0, head_dim, head_dim, None, None, 0.0, rot, True, table,
+                                   self.magnitude, ctx.positions, None, None, 1, None, None)
 
 
 @register_position_encoding("none")
