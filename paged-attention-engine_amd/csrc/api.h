@@ -81,6 +81,15 @@ int pae_attn_prefill_bf16(void* out, int64_t out_stride, const void* q, int64_t 
                           const void* v_cache, const int* tiles, int num_tiles, const int* positions,
                           const int* block_tables, int max_blocks, int bs, int nh, int nkv, int hd, float scale,
                           int window, hipStream_t stream);
+// the two above with capped scores (cap > 0: s <- cap tanh(s / cap)) and per-head sinks (float32 [nh] or null)
+int pae_attn_decode_capped_bf16(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* k_cache,
+                                const void* v_cache, const int* dec_work, int num_dec, const int* block_tables,
+                                int max_blocks, int bs, int nh, int nkv, int hd, float scale, int window, float cap,
+                                const float* sinks, void* part_acc, void* part_ml, hipStream_t stream);
+int pae_attn_prefill_capped_bf16(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* k_cache,
+                                 const void* v_cache, const int* tiles, int num_tiles, const int* positions,
+                                 const int* block_tables, int max_blocks, int bs, int nh, int nkv, int hd, float scale,
+                                 int window, float cap, const float* sinks, hipStream_t stream);
 // A decode step's layers as one resident kernel (see decode_program.hip).
 // A caller builds a list of phases in host memory with the put functions (each returns the bytes of
 // LDS a quad of four wavefronts needs for the phase, or a negative code), copies it to the device and

@@ -24,14 +24,21 @@ struct AttnState {
   float l[CT];             // this lane's share of the column's sum
 };
 
+// tanh by one exponential and one reciprocal (both hardware instructions, about a unit in the last place):
+// tanh(x) = 1 - 2 / (1 + e^(2x)); e^(2x) = inf gives 1, 0 gives -1.
+__device__ __forceinline__ float tanh_fast(float x) {
+  return 1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * (2.0f * LOG2E)));
+}
+
 // One 16-key tile.  `kp` points at key row 0 of the tile (row stride HD), `vp` at
 // value feature 0 of the tile's first key (feature stride `vstride` elements).
 // q[ct][j]: B operand of column tile ct for hd slice j.  pos/start: per lane's column.
-template <int HD, int CT>
+// CAPPED: scores are capped, s <- cap tanh(s / cap): `cap_log2` = cap log2(e), `scale_over_cap` = scale / cap.
+template <int HD, int CT, bool CAPPED = false>
 __device__ __forceinline__ void attn_tile(AttnState<HD, CT>& st, const bf16x8 (&kf)[HD / 32],
                                           const s16x4 (&vf)[HD / 16], const bf16x8 (&q)[CT][HD / 32],
                                           int key0, const int (&pos)[CT], const int (&start)[CT],
-                                          float scale_log2) {
+                                          float scale_log2, float cap_log2 = 0.f, float scale_over_cap = 0.f) {
   const int g4 = threadIdx.x % PAE_WAVE / 16;
 #pragma unroll
   for (int ct = 0; ct < CT; ++ct) {
@@ -42,7 +49,8 @@ __device__ __forceinline__ void attn_tile(AttnState<HD, CT>& st, const bf16x8 (&
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int key = key0 + 4 * g4 + i;
-      s[i] = (key <= pos[ct] && key >= start[ct]) ? s[i] * scale_log2 : -INFINITY;
+      const float scaled = CAPPED ? cap_log2 * tanh_fast(s[i] * scale_over_cap) : s[i] * scale_log2;
+      s[i] = (key <= pos[ct] && key >= start[ct]) ? scaled : -INFINITY;
       mx = fmaxf(mx, s[i]);
     }
     mx = fmaxf(mx, __shfl_xor(mx, 16, PAE_WAVE));

@@ -39,12 +39,13 @@
 // for every workgroup and cost more than the second launch.)
 //   part_acc[((token * nkv + kvh) * max_splits + split) * g + head in group][HD]
 //   part_ml [ ... same index ... ][2] = (maximum in log2 units, sum)
-template <int HD, int TPW>
+template <int HD, int TPW, bool CAPPED>
 __global__ __launch_bounds__(256) void attn_decode_kernel(
     float* __restrict__ part_acc, float* __restrict__ part_ml, int max_splits,
     const bf16_t* __restrict__ q, int64_t q_stride,
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache, const int4* __restrict__ dec_work,
-    const int* __restrict__ block_tables, int max_blocks, int bs, int nh, int nkv, float scale_log2, int window) {
+    const int* __restrict__ block_tables, int max_blocks, int bs, int nh, int nkv, float scale_log2, int window,
+    float cap_log2, float scale_over_cap) {
   constexpr int SPLIT = 64 * TPW;
   const int split = blockIdx.x, kvh = blockIdx.y;
   // one load brings the token's row, its position and its table row: a chain of three dependent
@@ -105,7 +106,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   for (int j = 0; j < TPW; ++j) {
     const int tile = tile_lo + wave + 4 * j;
     keys_to_mfma_order<HD>(kf[j]);  // in every lane of the wavefront, used or not
-    if (tile < tile_hi) attn_tile<HD, 1>(st, kf[j], vf[j], qf, tile * 16, pos, start, scale_log2);
+    if (tile < tile_hi)
+      attn_tile<HD, 1, CAPPED>(st, kf[j], vf[j], qf, tile * 16, pos, start, scale_log2, cap_log2, scale_over_cap);
   }
 
   // wavefronts 1..3 hand their state to wavefront 0 through LDS; every lane of a wavefront
@@ -160,7 +162,7 @@ template <int HD, int TPW>
 __global__ void attn_decode_merge_kernel(bf16_t* __restrict__ out, int64_t out_stride,
                                          const float* __restrict__ part_acc, const float* __restrict__ part_ml,
                                          int max_splits, const int4* __restrict__ dec_work, int nh, int nkv,
-                                         int window) {
+                                         int window, const float* __restrict__ sinks) {
   // blockDim = (items rounded up to wavefronts, G): the splits are dealt out to G groups of threads,
   // whose loads are all in flight together; group 0 then adds the groups' sums in group order.
   extern __shared__ float s_merge[];  // [G - 1][items][6]: four sums, maximum, sum of weights
@@ -205,6 +207,13 @@ __global__ void attn_decode_merge_kernel(bf16_t* __restrict__ out, int64_t out_s
     l = l * f_old + ls * f;
     m = m_new;
   }
+  if (sinks) {  // the head's sink joins the denominator: exp(sink) without a value
+    const float sink = sinks[kvh * g + c] * LOG2E;
+    const float m_new = fmaxf(m, sink);
+    const float f_old = exp2f(m - m_new);
+    a = a * f_old;
+    l = l * f_old + exp2f(sink - m_new);
+  }
   const float inv = 1.0f / l;
   s16x4 w;
 #pragma unroll
@@ -245,12 +254,12 @@ __device__ __forceinline__ bf16x8 quad_to_mfma_order(bf16x8 x, int fetch_from) {
 // tiles[t] = (table row of the sequence, first flat token, number of tokens <= 64); blockIdx.z picks
 // the part of 16 CT tokens of the run that this workgroup takes.
 // BS: the page size if it is 16 (the value rows' offsets are then constants), or 0 for any other.
-template <int HD, int CT, int BS>
+template <int HD, int CT, int BS, bool CAPPED>
 __global__ __launch_bounds__(256, 1) void attn_prefill_split_kernel(
     bf16_t* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ q, int64_t q_stride,
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache, const int* __restrict__ tiles,
     const int* __restrict__ positions, const int* __restrict__ block_tables, int max_blocks, int bs, int nh,
-    int nkv, float scale_log2, int window) {
+    int nkv, float scale_log2, int window, float cap_over_scale, float scale_over_cap, const float* __restrict__ sinks) {
   constexpr int UNIT = 32, TOK = 16 * CT;
   if (BS) bs = BS;
   __shared__ float s_acc[3][HD / 16][4][PAE_WAVE];
@@ -372,6 +381,14 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_split_kernel(
             s[ct][p] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[p][j], qf[ct][j], s[ct][p], 0, 0, 0);
         }
     }
+    if (CAPPED) {  // s <- (cap / scale) tanh(s scale / cap): what follows multiplies by the scale as before
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+        for (int p = 0; p < 2; ++p)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) s[ct][p][i] = cap_over_scale * tanh_fast(s[ct][p][i] * scale_over_cap);
+    }
     if (more) load_keys(key0 + 4 * UNIT);  // into the registers the first product has just read
     if (!(key0 + UNIT - 1 <= pos0 && key0 >= last_start)) {  // some key is hidden from some token of the run
 #pragma unroll
@@ -473,8 +490,11 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_split_kernel(
       float m = ref[ct];
 #pragma unroll
       for (int w = 0; w < 3; ++w) m = fmaxf(m, s_ml[w][0][lane]);
+      const float sink = sinks ? sinks[head] * LOG2E : 0.f;
+      if (sinks) m = fmaxf(m, sink);
       const float own = exp2f(ref[ct] - m);
       float sum = l[ct] * own;
+      if (sinks) sum += exp2f(sink - m);  // the head's sink joins the denominator without a value
       float scale_w[3];
 #pragma unroll
       for (int w = 0; w < 3; ++w) {
@@ -534,10 +554,12 @@ extern "C" int pae_attn_decode_split() { return 64 * DECODE_TPW; }
 // 16 bytes each, 16-byte aligned.
 // Workspace: part_acc holds num_dec * nh * max_splits * hd floats, part_ml num_dec * nh * max_splits * 2,
 // max_splits = ceil(max_blocks * bs / pae_attn_decode_split()).
-extern "C" int pae_attn_decode_bf16(void* out, int64_t out_stride, const void* q, int64_t q_stride,
+// `cap` > 0: scores are capped, s <- cap tanh(s / cap); `sinks` (float32 [nh], or null): one number per query
+// head that joins its softmax's denominator as exp(sink).
+extern "C" int pae_attn_decode_capped_bf16(void* out, int64_t out_stride, const void* q, int64_t q_stride,
                                     const void* k_cache, const void* v_cache, const int* dec_work, int num_dec,
                                     const int* block_tables, int max_blocks, int bs, int nh, int nkv, int hd, float scale, int window,
-                                    void* part_acc, void* part_ml, hipStream_t stream) {
+                                    float cap, const float* sinks, void* part_acc, void* part_ml, hipStream_t stream) {
   if (int rc = check_common("attn_decode", nh, nkv, hd, bs, max_blocks, window)) return rc;
   PAE_REQUIRE(num_dec <= 65535 && nkv <= 65535, "attn_decode: grid too large");
   if (num_dec <= 0) return 0;
@@ -554,26 +576,43 @@ extern "C" int pae_attn_decode_bf16(void* out, int64_t out_stride, const void* q
   if (merge_groups < 1) merge_groups = 1;
   PAE_REQUIRE(merge_x <= 1024, "attn_decode: %d heads of %d features per key/value head exceed the merge's workgroup", nh / nkv, hd);
   const size_t merge_lds = (size_t)(merge_groups - 1) * merge_items * 6 * sizeof(float);
-#define CALL(HD)                                                                                            \
-  attn_decode_kernel<HD, DECODE_TPW><<<grid, 256, (size_t)3 * (HD / 4 + 2) * PAE_WAVE * sizeof(float), stream>>>( \
+  PAE_REQUIRE(cap >= 0.f, "attn_decode: negative score cap %g", (double)cap);
+  const float cap_log2 = cap * LOG2E, scale_over_cap = cap > 0.f ? scale / cap : 0.f;
+#define CALL_CAPPED(HD, CAPPED)                                                                              \
+  attn_decode_kernel<HD, DECODE_TPW, CAPPED><<<grid, 256, (size_t)3 * (HD / 4 + 2) * PAE_WAVE * sizeof(float), stream>>>( \
       (float*)part_acc, (float*)part_ml, max_splits, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache,     \
       (const bf16_t*)v_cache, (const int4*)dec_work, block_tables, max_blocks, bs, nh, nkv, scale_log2, \
-      window);                                                                                               \
+      window, cap_log2, scale_over_cap)
+#define CALL(HD)                                                                                            \
+  if (cap > 0.f) {                                                                                          \
+    CALL_CAPPED(HD, true);                                                                                  \
+  } else {                                                                                                  \
+    CALL_CAPPED(HD, false);                                                                                 \
+  }                                                                                                         \
   attn_decode_merge_kernel<HD, DECODE_TPW><<<merge_grid, dim3(merge_x, merge_groups), merge_lds, stream>>>( \
       (bf16_t*)out, out_stride, (const float*)part_acc, (const float*)part_ml, max_splits, (const int4*)dec_work, \
-      nh, nkv, window)
+      nh, nkv, window, sinks)
   FOR_HEAD_DIM(hd, CALL)
 #undef CALL
+#undef CALL_CAPPED
   return pae_check_launch("attn_decode");
+}
+
+extern "C" int pae_attn_decode_bf16(void* out, int64_t out_stride, const void* q, int64_t q_stride,
+                                    const void* k_cache, const void* v_cache, const int* dec_work, int num_dec,
+                                    const int* block_tables, int max_blocks, int bs, int nh, int nkv, int hd, float scale, int window,
+                                    void* part_acc, void* part_ml, hipStream_t stream) {
+  return pae_attn_decode_capped_bf16(out, out_stride, q, q_stride, k_cache, v_cache, dec_work, num_dec, block_tables,
+                                     max_blocks, bs, nh, nkv, hd, scale, window, 0.f, nullptr, part_acc, part_ml, stream);
 }
 
 // tiles[t] = (table row of the sequence, first flat token, number of tokens <= 64), heaviest runs
 // first: workgroups start in the order of the grid, and the last to finish sets the time.
-extern "C" int pae_attn_prefill_bf16(void* out, int64_t out_stride, const void* q, int64_t q_stride,
+extern "C" int pae_attn_prefill_capped_bf16(void* out, int64_t out_stride, const void* q, int64_t q_stride,
                                           const void* k_cache, const void* v_cache, const int* tiles,
                                           int num_tiles, const int* positions, const int* block_tables,
                                           int max_blocks, int bs, int nh, int nkv, int hd, float scale, int window,
-                                          hipStream_t stream) {
+                                          float cap, const float* sinks, hipStream_t stream) {
   if (int rc = check_common("attn_prefill", nh, nkv, hd, bs, max_blocks, window)) return rc;
   PAE_REQUIRE(num_tiles <= 65535, "attn_prefill: %d runs exceed the grid", num_tiles);
   if (num_tiles <= 0) return 0;
@@ -583,10 +622,19 @@ extern "C" int pae_attn_prefill_bf16(void* out, int64_t out_stride, const void* 
   // workgroups, each with half the arithmetic per 32 keys (1.5B heads: 512 tokens 16.4 -> 12.1 us, 1,024
   // tokens 22.0 -> 19.3; from 2,048 tokens on, 384 workgroups, four tiles are ahead: 40.5 against 47.0 us).
   const bool halves = (int64_t)nh * num_tiles <= 256;
-#define LAUNCH_CT(HD, CT, BS)                                                                                  \
-  attn_prefill_split_kernel<HD, CT, BS><<<dim3(nh, num_tiles, 4 / CT), 256, 0, stream>>>(                      \
+  PAE_REQUIRE(cap >= 0.f && (cap == 0.f || scale > 0.f), "attn_prefill: bad score cap %g (scale %g)", (double)cap, (double)scale);
+  const float cap_over_scale = cap > 0.f ? cap / scale : 0.f, scale_over_cap = cap > 0.f ? scale / cap : 0.f;
+#define LAUNCH_CAPPED(HD, CT, BS, CAPPED)                                                                      \
+  attn_prefill_split_kernel<HD, CT, BS, CAPPED><<<dim3(nh, num_tiles, 4 / CT), 256, 0, stream>>>(              \
       (bf16_t*)out, out_stride, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache,    \
-      tiles, positions, block_tables, max_blocks, bs, nh, nkv, scale_log2, window)
+      tiles, positions, block_tables, max_blocks, bs, nh, nkv, scale_log2, window, cap_over_scale,             \
+      scale_over_cap, sinks)
+#define LAUNCH_CT(HD, CT, BS)           \
+  if (cap > 0.f) {                      \
+    LAUNCH_CAPPED(HD, CT, BS, true);    \
+  } else {                              \
+    LAUNCH_CAPPED(HD, CT, BS, false);   \
+  }
 #define LAUNCH(HD, BS)                  \
   if (HD > 128 || halves) {             \
     LAUNCH_CT(HD, 2, BS);               \
@@ -603,5 +651,14 @@ extern "C" int pae_attn_prefill_bf16(void* out, int64_t out_stride, const void* 
 #undef CALL
 #undef LAUNCH
 #undef LAUNCH_CT
+#undef LAUNCH_CAPPED
   return pae_check_launch("attn_prefill");
+}
+
+extern "C" int pae_attn_prefill_bf16(void* out, int64_t out_stride, const void* q, int64_t q_stride,
+                                     const void* k_cache, const void* v_cache, const int* tiles, int num_tiles,
+                                     const int* positions, const int* block_tables, int max_blocks, int bs, int nh,
+                                     int nkv, int hd, float scale, int window, hipStream_t stream) {
+  return pae_attn_prefill_capped_bf16(out, out_stride, q, q_stride, k_cache, v_cache, tiles, num_tiles, positions,
+                                      block_tables, max_blocks, bs, nh, nkv, hd, scale, window, 0.f, nullptr, stream);
 }

@@ -82,6 +82,8 @@ def _declare(lib) -> None:
         "pae_sample_static_prepare": [],
         "pae_attn_decode_bf16": [P, L, P, L, P, P, P, I, P, I, I, I, I, I, F, I, P, P, P],
         "pae_attn_decode_split": [],
+        "pae_attn_decode_capped_bf16": [P, L, P, L, P, P, P, I, P, I, I, I, I, I, F, I, F, P, P, P, P],
+        "pae_attn_prefill_capped_bf16": [P, L, P, L, P, P, P, I, P, P, I, I, I, I, I, F, I, F, P, P],
         "pae_attn_prefill_bf16": [P, L, P, L, P, P, P, I, P, P, I, I, I, I, I, F, I, P],
         "pae_program_phase_bytes": [],
         "pae_program_barrier_bytes": [],
@@ -1032,11 +1034,15 @@ def mfma_attention_supported(dtype: torch.dtype, nh: int, nkv: int, hd: int, bs:
 
 def attn_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                 dec_work: torch.Tensor, block_tables: torch.Tensor, nh: int, nkv: int, hd: int, scale: float,
-                window: int) -> None:
+                window: int, softcap: float = 0.0, sinks: Optional[torch.Tensor] = None) -> None:
     """Attention of the single new token of each sequence listed in `dec_work` over that sequence's
     cached keys: split over the keys, then merged.  dec_work[i] = (flat row of the token, its
-    position, row of its sequence in `block_tables`, 0)."""
-    _gpu(out, q, k_cache, v_cache, dec_work, block_tables)
+    position, row of its sequence in `block_tables`, 0).  `softcap` > 0 caps the scores
+    (s <- softcap tanh(s / softcap)); `sinks` (float32 [nh]) join each head's softmax denominator."""
+    _gpu(out, q, k_cache, v_cache, dec_work, block_tables, sinks)
+    wide = bool(softcap) or sinks is not None
+    if sinks is not None:
+        assert sinks.dtype == torch.float32 and sinks.numel() == nh and sinks.is_contiguous()
     bs = k_cache.shape[2]
     assert q.dtype == torch.bfloat16 == out.dtype == k_cache.dtype and q.stride(1) == 1 and out.stride(1) == 1
     assert q.shape[1] >= nh * hd and out.shape[1] >= nh * hd and out.shape[0] == q.shape[0]
@@ -1050,6 +1056,13 @@ def attn_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cac
     max_splits = -(-block_tables.shape[1] * bs // library().pae_attn_decode_split())
     part_acc = torch.empty((n * nh * max_splits, hd), dtype=torch.float32, device=q.device)
     part_ml = torch.empty((n * nh * max_splits, 2), dtype=torch.float32, device=q.device)
+    if wide:
+        _not_while_recording("attn_decode with a score cap or sinks")
+        _check(library().pae_attn_decode_capped_bf16(
+            out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
+            dec_work.data_ptr(), n, block_tables.data_ptr(), block_tables.shape[1], bs, nh, nkv, hd, float(scale),
+            int(window), float(softcap), _ptr(sinks), part_acc.data_ptr(), part_ml.data_ptr(), _stream()))
+        return
     if _RECORDING is not None:
         _RECORDING.room(2)  # the splits' partial results, then their merge
         code = library().pae_program_put_attention(
@@ -1070,13 +1083,16 @@ PREFILL_TILE = 64  # tokens per run of the prefill attention kernel (one workgro
 
 def attn_prefill(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                  tiles: torch.Tensor, positions: torch.Tensor, block_tables: torch.Tensor,
-                 nh: int, nkv: int, hd: int, scale: float, window: int) -> None:
+                 nh: int, nkv: int, hd: int, scale: float, window: int, softcap: float = 0.0,
+                 sinks: Optional[torch.Tensor] = None) -> None:
     """Attention of runs of consecutive tokens; tiles[t] = (table row of the sequence, first
     flat token, number of tokens <= PREFILL_TILE).  One workgroup per run and head, whose
     wavefronts share out the keys; workgroups start in the order of `tiles`, so the runs with
-    the most keys should come first."""
+    the most keys should come first.  `softcap` and `sinks` as in `attn_decode`."""
     _not_while_recording("attn_prefill")
-    _gpu(out, q, k_cache, v_cache, tiles, positions, block_tables)
+    _gpu(out, q, k_cache, v_cache, tiles, positions, block_tables, sinks)
+    if sinks is not None:
+        assert sinks.dtype == torch.float32 and sinks.numel() == nh and sinks.is_contiguous()
     bs = k_cache.shape[2]
     assert q.dtype == torch.bfloat16 == out.dtype == k_cache.dtype and q.stride(1) == 1 and out.stride(1) == 1
     assert q.shape[1] >= nh * hd and out.shape[1] >= nh * hd and out.shape[0] == q.shape[0]
@@ -1084,10 +1100,10 @@ def attn_prefill(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_ca
     assert tiles.dtype == torch.int32 and tiles.dim() == 2 and tiles.shape[1] == 3 and tiles.is_contiguous()
     assert positions.dtype == torch.int32 and positions.numel() == q.shape[0]
     assert block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous()
-    _check(library().pae_attn_prefill_bf16(
+    _check(library().pae_attn_prefill_capped_bf16(
         out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
         tiles.data_ptr(), tiles.shape[0], positions.data_ptr(), block_tables.data_ptr(), block_tables.shape[1],
-        bs, nh, nkv, hd, float(scale), int(window), _stream()))
+        bs, nh, nkv, hd, float(scale), int(window), float(softcap), _ptr(sinks), _stream()))
 
 
 def sample(tokens: torch.Tensor, logits: torch.Tensor, temperature: Optional[torch.Tensor],

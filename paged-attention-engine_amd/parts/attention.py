@@ -56,6 +56,23 @@ def attention_work_lists(shape: StepShape):
     return {"decode_work": (decode_work, 4), "prefill_tiles": ([x for _, tile in runs for x in tile], 3)}
 
 
+def attend_paged(attn, q, k_cache, v_cache, positions, tok_seq, table, work, num_heads: int, num_kv_heads: int,
+                 head_dim: int, value_dim: int, scale: float, window: int, softcap: float, sinks) -> None:
+    """Attention of a step's queries over the paged cache into `attn`: with `work` (the device lists of
+    `attention_work_lists`) on the matrix cores, single tokens by the decode kernel and runs of tokens by
+    the prefill kernel; without, by the kernel that takes any shape and precision."""
+    if work is not None:
+        geometry = (num_heads, num_kv_heads, head_dim, scale, window, softcap, sinks)
+        decode_work, prefill_tiles = work["decode_work"], work["prefill_tiles"]
+        if decode_work.numel():
+            K.attn_decode(attn, q, k_cache, v_cache, decode_work, table, *geometry)
+        if prefill_tiles.numel():
+            K.attn_prefill(attn, q, k_cache, v_cache, prefill_tiles, positions, table, *geometry)
+    else:
+        K.paged_attention_capped(attn, q, k_cache, v_cache, positions, tok_seq, table, num_heads, num_kv_heads,
+                                 head_dim, value_dim, scale, window, softcap, sinks)
+
+
 @register_mixer("attention")
 class PagedAttention(Part):
     takes_owed_rows = True
@@ -82,7 +99,7 @@ class PagedAttention(Part):
 
     @property
     def graph_max_rows(self):
-        return rows_a_graph_may_hold(self.dtype, self.spec.hidden_size, self.spec.num_heads * self.spec.head_dim)
+        return rows_a_graph_may_hold(self.dtype, self.spec.hidden_size, self.spec.num_heads * self.spec.v_dim)
 
     def decode_fusable(self, rows: int, block_size: int) -> bool:
         """One token a sequence, few rows: the fused projection, the decode attention and the output
@@ -103,10 +120,11 @@ class PagedAttention(Part):
 
     def _matrix_cores(self, block_size: int) -> bool:
         s = self.spec
-        return K.mfma_attention_supported(self.dtype, s.num_heads, s.num_kv_heads, s.head_dim, block_size)
+        return (s.v_dim == s.head_dim
+                and K.mfma_attention_supported(self.dtype, s.num_heads, s.num_kv_heads, s.head_dim, block_size))
 
     def step_lists_key(self, block_size: int):
-        return WORK_LISTS if self.spec.plain and self._matrix_cores(block_size) else None
+        return WORK_LISTS if self._matrix_cores(block_size) else None
 
     def step_lists(self, shape: StepShape):
         return attention_work_lists(shape)
@@ -206,9 +224,9 @@ class PagedAttention(Part):
                                ctx.tok_seq if nkv else None, table if nkv else None, ctx.cache.block_size,
                                k_cache, v_cache)
         attn = torch.empty((qkv.shape[0], s.num_heads * s.v_dim), dtype=qkv.dtype, device=qkv.device)
-        K.paged_attention_capped(attn, qkv, pages["k"], pages["v"], ctx.positions, ctx.tok_seq, table, s.num_heads,
-                                 s.num_kv_heads, s.head_dim, s.v_dim, s.scale, s.window or 0, s.softcap or 0.0,
-                                 self.sinks)
+        work = ctx.memo.get(WORK_LISTS) if self._matrix_cores(ctx.cache.block_size) else None
+        attend_paged(attn, qkv, pages["k"], pages["v"], ctx.positions, ctx.tok_seq, table, work, s.num_heads,
+                     s.num_kv_heads, s.head_dim, s.v_dim, s.scale, s.window or 0, s.softcap or 0.0, self.sinks)
         return self.out.branch(attn, ctx.sink)
 
     def forward(self, ctx, x):

@@ -34,6 +34,29 @@ import torch
 
 DELTA_UNIT_EPS = 1e-6  # inside the root when q and k are made unit vectors
 
+# What reduced precision alone does to the logits: with STORAGE set to a type (torch.bfloat16), every
+# matrix product reads operands rounded to it and its result is rounded to it, and so are the rotated
+# queries and keys, the values, and the activations handed from one product to the next; sums, norms,
+# softmax, the recurrence and the residual stay in the working precision.  A test of a reduced-precision
+# engine measures its error against the error of this.
+STORAGE = None
+# (generator, relative size): every product's sums are moved by that much at random before they are
+# rounded, as another order of adding moves them (a fraction of a unit in the last place of the
+# storage type): two kernels that are both right differ by this, and a model that is touchy
+# somewhere (a norm right after a sum that nearly cancels) turns it into visible differences.
+JITTER = None
+
+
+def stored(x: torch.Tensor) -> torch.Tensor:
+    return x if STORAGE is None else x.to(STORAGE).to(x.dtype)
+
+
+def product(h: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    y = stored(h) @ weight.T
+    if JITTER is not None:
+        y = y * (1.0 + JITTER[1] * torch.randn(y.shape, generator=JITTER[0], dtype=y.dtype))
+    return stored(y)
+
 
 def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     return x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps) * weight
@@ -91,31 +114,42 @@ def rotate_interleaved(x: torch.Tensor, positions: torch.Tensor, rot: dict, angl
 # --------------------------------------------------------------------------- mixers
 
 
-def attention_mixer(h: torch.Tensor, w: dict, prefix: str, mix: dict, eps: float, angle_dtype=None) -> torch.Tensor:
-    T = h.shape[0]
-    H, G, D, V = int(mix["heads"]), int(mix["kv_heads"]), int(mix["dim"]), int(mix["vdim"])
-    q = rms_norm(h @ w[prefix + "q"].T, w[prefix + "q.norm"], eps).view(T, H, D)
-    k = rms_norm(h @ w[prefix + "k"].T, w[prefix + "k.norm"], eps).view(T, G, D)
-    v = (h @ w[prefix + "v"].T).view(T, G, V)
-    positions = torch.arange(T)
-    if mix.get("rot"):
-        q = rotate_interleaved(q, positions, mix["rot"], angle_dtype)
-        k = rotate_interleaved(k, positions, mix["rot"], angle_dtype)
-    out = torch.zeros(T, H, V, dtype=h.dtype)
-    cap = mix.get("softcap")
+def attend(q, k, v, scale: float, cap, sinks, positions=None) -> torch.Tensor:
+    """q [T, H, D], k [T, G, D], v [T, G, V], sinks [H] or None -> [T, H, V]; query t sees keys 0..t."""
+    T, H = q.shape[0], q.shape[1]
+    G, V = k.shape[1], v.shape[2]
+    positions = torch.arange(T) if positions is None else positions
     causal = positions[None, :] <= positions[:, None]
+    out = torch.zeros(T, H, V, dtype=q.dtype)
     for head in range(H):
         g = head // (H // G)
-        s = (q[:, head] @ k[:, g].T) * float(mix["scale"])
+        s = (q[:, head] @ k[:, g].T) * float(scale)
         if cap:
             s = float(cap) * torch.tanh(s / float(cap))
         s = s.masked_fill(~causal, -math.inf)
-        sink = w[prefix + "sink"][head]
-        top = torch.maximum(s.max(dim=-1, keepdim=True).values, sink)
+        top = s.max(dim=-1, keepdim=True).values
+        if sinks is not None:
+            top = torch.maximum(top, sinks[head])
         e = torch.exp(s - top)
-        denom = e.sum(-1, keepdim=True) + torch.exp(sink - top)
+        denom = e.sum(-1, keepdim=True)
+        if sinks is not None:
+            denom = denom + torch.exp(sinks[head] - top)
         out[:, head] = (e / denom) @ v[:, g]
-    return out.reshape(T, H * V) @ w[prefix + "o"].T
+    return out
+
+
+def attention_mixer(h: torch.Tensor, w: dict, prefix: str, mix: dict, eps: float, angle_dtype=None) -> torch.Tensor:
+    T = h.shape[0]
+    H, G, D, V = int(mix["heads"]), int(mix["kv_heads"]), int(mix["dim"]), int(mix["vdim"])
+    q = rms_norm(product(h, w[prefix + "q"]), w[prefix + "q.norm"], eps).view(T, H, D)
+    k = rms_norm(product(h, w[prefix + "k"]), w[prefix + "k.norm"], eps).view(T, G, D)
+    v = product(h, w[prefix + "v"]).view(T, G, V)
+    positions = torch.arange(T)
+    if mix.get("rot") and int(mix["rot"].get("dims", 0)):
+        q = rotate_interleaved(q, positions, mix["rot"], angle_dtype)
+        k = rotate_interleaved(k, positions, mix["rot"], angle_dtype)
+    out = attend(stored(q), stored(k), v, mix["scale"], mix.get("softcap"), w[prefix + "sink"])
+    return product(out.reshape(T, H * V), w[prefix + "o"])
 
 
 def causal_conv_silu(x: torch.Tensor, taps: torch.Tensor) -> torch.Tensor:
@@ -133,30 +167,45 @@ def unit(x: torch.Tensor) -> torch.Tensor:
     return x / torch.sqrt(x.pow(2).sum(-1, keepdim=True) + DELTA_UNIT_EPS)
 
 
-def delta_mixer(h: torch.Tensor, w: dict, prefix: str, mix: dict, eps: float) -> torch.Tensor:
-    T = h.shape[0]
-    H, G, D, V = int(mix["heads"]), int(mix["kv_heads"]), int(mix["dim"]), int(mix["vdim"])
-    q = unit(causal_conv_silu(h @ w[prefix + "q"].T, w[prefix + "q.conv"]).view(T, G, D)) * D ** -0.5
-    k = unit(causal_conv_silu(h @ w[prefix + "k"].T, w[prefix + "k.conv"]).view(T, G, D))
-    v = causal_conv_silu(h @ w[prefix + "v"].T, w[prefix + "v.conv"]).view(T, H, V)
-    beta = torch.sigmoid(h @ w[prefix + "b"].T)                                              # [T, H]
-    decay = torch.exp(-torch.exp(w[prefix + "A_log"]) * softplus(h @ w[prefix + "a"].T + w[prefix + "dt_bias"]))
-    gate = silu(h @ w[prefix + "g"].T).view(T, H, V)
-    out = torch.zeros(T, H, V, dtype=h.dtype)
+def delta_recurrence(q, k, v, beta, decay) -> torch.Tensor:
+    """q, k [T, G, D] (already unit vectors), v [T, H, V], beta, decay [T, H] -> o [T, H, V].
+    Per head:  S <- decay S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q,  S = 0 before the first token."""
+    T, G, D = q.shape
+    H, V = v.shape[1], v.shape[2]
+    out = torch.zeros(T, H, V, dtype=q.dtype)
     for head in range(H):
         g = head // (H // G)
-        S = torch.zeros(D, V, dtype=h.dtype)
+        S = torch.zeros(D, V, dtype=q.dtype)
         for t in range(T):
             S = decay[t, head] * S
             u = beta[t, head] * (v[t, head] - S.T @ k[t, g])
             S = S + torch.outer(k[t, g], u)
             out[t, head] = S.T @ q[t, g]
-    out = out / torch.sqrt(out.pow(2).mean(-1, keepdim=True) + eps) * w[prefix + "norm"] * gate
-    return out.reshape(T, H * V) @ w[prefix + "o"].T
+    return out
+
+
+def delta_core(qp, kp, vp, gate_p, b_p, a_p, q_conv, k_conv, v_conv, a_log, dt_bias, norm_w, G, H, D, V, eps):
+    """Everything of the delta mixer between its input projections and its output projection."""
+    T = qp.shape[0]
+    q = unit(causal_conv_silu(qp, q_conv).view(T, G, D)) * D ** -0.5
+    k = unit(causal_conv_silu(kp, k_conv).view(T, G, D))
+    v = causal_conv_silu(vp, v_conv).view(T, H, V)
+    beta = torch.sigmoid(b_p)
+    decay = torch.exp(-torch.exp(a_log) * softplus(a_p + dt_bias))
+    out = delta_recurrence(q, k, v, beta, decay)
+    out = out / torch.sqrt(out.pow(2).mean(-1, keepdim=True) + eps) * norm_w * silu(gate_p).view(T, H, V)
+    return out.reshape(T, H * V)
+
+
+def delta_mixer(h: torch.Tensor, w: dict, prefix: str, mix: dict, eps: float) -> torch.Tensor:
+    H, G, D, V = int(mix["heads"]), int(mix["kv_heads"]), int(mix["dim"]), int(mix["vdim"])
+    out = delta_core(*(product(h, w[prefix + name]) for name in "qkvgba"), w[prefix + "q.conv"], w[prefix + "k.conv"],
+                     w[prefix + "v.conv"], w[prefix + "A_log"], w[prefix + "dt_bias"], w[prefix + "norm"], G, H, D, V, eps)
+    return product(out, w[prefix + "o"])
 
 
 def feed_forward(h: torch.Tensor, w: dict, prefix: str) -> torch.Tensor:
-    return gelu_erf(h @ w[prefix + "up"].T) @ w[prefix + "down"].T
+    return product(gelu_erf(product(h, w[prefix + "up"])), w[prefix + "down"])
 
 
 # --------------------------------------------------------------------------- model
@@ -180,7 +229,7 @@ def forward(weights: dict, cfg: dict, tokens, dtype=torch.float64, angle_dtype=N
         if layer.get("mlp") is not None:
             x = x + m * rms_norm(feed_forward(x, w, p + "mlp."), w[p + "norm2"], eps)
         kept.append(x)
-    logits = (rms_norm(x, w["final.norm"], eps) @ w["embed"].T) * float(cfg["logit_scale"])
+    logits = (stored(rms_norm(x, w["final.norm"], eps)) @ w["embed"].T) * float(cfg["logit_scale"])
     return (logits, torch.stack(kept)) if keep_layers else logits
 
 
