@@ -56,6 +56,59 @@ OTHER_SHAPES = {
                 num_key_value_heads=8, intermediate_size=29568, vocab_size=152064, rms_norm_eps=1e-5,
                 tie_word_embeddings=False),
 }
+
+
+def danonex_shape(shape: dict, layers: int) -> dict:
+    """A Danonex configuration with the layer sizes of the Qwen2.5 shape `shape`: the same width, head
+    counts and head size in its attention layers (values as wide as keys, capped scores, stretched
+    rotation, sinks), the same heads in its recurrent layers (half as many query/key heads, convolutions
+    of four taps), the same feed-forward width (ungated), the same vocabulary; three attention layers to
+    one recurrent layer, every layer with a feed-forward."""
+    heads, kv, hd = shape["num_attention_heads"], shape["num_key_value_heads"], shape["head_dim"]
+    rot = {"base": float(shape["rope_theta"]), "dims": hd,
+           "scaling": {"factor": 4.0, "original": 8192, "fast": 32.0, "slow": 1.0}}
+    attention = {"type": "attention", "mlp": {"kind": "dense", "ff": shape["intermediate_size"]},
+                 "mixer": {"heads": heads, "kv_heads": kv, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "softcap": 50.0,
+                           "rot": rot}}
+    recurrent = {"type": "delta", "mlp": {"kind": "dense", "ff": shape["intermediate_size"]},
+                 "mixer": {"heads": heads, "kv_heads": max(1, heads // 2), "dim": hd, "vdim": hd, "conv": 4}}
+    return {"architecture": "Danonex", "vocab": shape["vocab_size"], "width": shape["hidden_size"],
+            "norm": {"eps": shape["rms_norm_eps"]}, "residual_mult": 0.7, "logit_scale": 0.25,
+            "layers": [recurrent if i % 4 == 1 else attention for i in range(layers)]}
+
+
+def design_run(args, shape: dict) -> int:
+    """`--design danonex`: decode steps (batch 1, 8, 64 at the context asked for) and a 2,048-token
+    prefill of a Danonex model with the shape's layer sizes, and beside each the same measurement of the
+    Qwen2.5 shape with the same number of layers.  One JSON line."""
+    import torch
+
+    layers = args.layers or 8
+    record = {"metric": f"Danonex beside Qwen2.5 at the {args.model} layer sizes, {layers} layers: decode tok/s and "
+                        f"prefill tok/s", "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+              "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "context": args.ctx,
+              "data": "synthetic: seeded uniform token ids, random weights N(0, 0.02)", "designs": {}}
+    configs = {"danonex": danonex_shape(shape, layers), "qwen2": dict(shape, num_hidden_layers=layers)}
+    for name, cfg in configs.items():
+        model = build_model(cfg, args.dtype)
+        vocab_cfg = {"vocab_size": shape["vocab_size"], "max_position_embeddings": shape.get("max_position_embeddings")}
+        out = {}
+        for batch in (1, 8, 64):
+            step_s, spread, _, _, recordings = decode_run(model, vocab_cfg, batch, args.ctx, args.steps, args.warmup)
+            out[f"decode_b{batch}"] = {"tokens_per_s": round(batch / step_s, 1), "ms_per_step": round(step_s * 1e3, 4),
+                                       "range_ms": round(spread * 1e3, 4), "graph_recordings": recordings}
+        for T in (2048, 8192):
+            pre_s, pre_range = prefill_run(model, vocab_cfg, T)
+            out[f"prefill_{T}"] = {"tokens_per_s": round(T / pre_s, 1), "ms": round(pre_s * 1e3, 3),
+                                   "range_ms": round(pre_range * 1e3, 3)}
+        record["designs"][name] = out
+        del model
+        torch.cuda.empty_cache()
+    record["value"] = record["designs"]["danonex"]["decode_b8"]["tokens_per_s"]
+    print(json.dumps(record))
+    return 0
+
+
 HBM_PEAK_GBS = 8000.0
 PEAK_FLOPS = {"bfloat16": 2.5e15, "float32": 157.3e12}
 
@@ -284,6 +337,10 @@ def main() -> int:
     parser.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill runs")
     parser.add_argument("--prefill-only", action="store_true", help="time the 2,048-token prefill alone (for profiles)")
+    parser.add_argument("--design", choices=("qwen2", "danonex"), default="qwen2",
+                        help="danonex: a Danonex model with the shape's layer sizes (8 layers unless --layers says "
+                             "otherwise) beside the Qwen2.5 shape with as many layers: decode at batch 1, 8, 64 and "
+                             "prefills of 2,048 and 8,192 tokens")
     args = parser.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU only: this engine has no multi-GPU path (run with --gpus 1)")
@@ -294,6 +351,12 @@ def main() -> int:
         print("bench.py needs a GPU", file=sys.stderr)
         return 1
     shape = QWEN25_1P5B if args.model == "1.5b" else OTHER_SHAPES[args.model]
+    if args.design == "danonex":
+        try:
+            return design_run(args, shape)
+        except (Refused, Unresolved) as err:
+            print(f"bench.py: {err}")
+            return 2
     args.full_layers = shape["num_hidden_layers"]
     args.layers = args.layers or args.full_layers
     args.shape_name = f"Qwen2.5-{args.model.upper()} shape"

@@ -62,6 +62,68 @@ __global__ __launch_bounds__(256) void norm_scale_add_kernel(float* __restrict__
   }
 }
 
+// Widths that are multiples of four up to 4,096: a thread owns up to four chunks of four columns, and
+// everything it needs (the branch's row, the residual, the weight) is asked for at once, before the
+// sum of squares is known: one trip to memory, then arithmetic, then the stores.
+template <typename T>
+__global__ __launch_bounds__(256) void norm_scale_add_vec_kernel(float* __restrict__ residual, const void* __restrict__ y,
+                                                                 int parts, int64_t part_stride,
+                                                                 const void* __restrict__ weight, int w_is_f32, float eps,
+                                                                 float scale, T* __restrict__ next, int hidden) {
+  __shared__ float scratch[4];
+  const int64_t base = (int64_t)blockIdx.x * hidden;
+  const int nvec = hidden / 4;
+  float yv[4][4], rv[4][4], wv[4][4];
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const int v4 = threadIdx.x + 256 * c;
+    if (v4 >= nvec) break;
+    if (parts == 0) {
+      if (sizeof(T) == 4) {
+        const float4 a = reinterpret_cast<const float4*>((const float*)y + base)[v4];
+        yv[c][0] = a.x; yv[c][1] = a.y; yv[c][2] = a.z; yv[c][3] = a.w;
+      } else {
+        const uint2 a = reinterpret_cast<const uint2*>((const bf16_t*)y + base)[v4];
+        yv[c][0] = __uint_as_float(a.x << 16); yv[c][1] = __uint_as_float(a.x & 0xffff0000u);
+        yv[c][2] = __uint_as_float(a.y << 16); yv[c][3] = __uint_as_float(a.y & 0xffff0000u);
+      }
+    } else {
+      yv[c][0] = yv[c][1] = yv[c][2] = yv[c][3] = 0.f;
+      for (int p = 0; p < parts; ++p) {  // partial sums are added in order
+        const float4 a = reinterpret_cast<const float4*>((const float*)y + p * part_stride + base)[v4];
+        yv[c][0] += a.x; yv[c][1] += a.y; yv[c][2] += a.z; yv[c][3] += a.w;
+      }
+    }
+    const float4 r = reinterpret_cast<const float4*>(residual + base)[v4];
+    rv[c][0] = r.x; rv[c][1] = r.y; rv[c][2] = r.z; rv[c][3] = r.w;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      wv[c][i] = load_param(weight, w_is_f32, 4 * v4 + i);
+      ss = fmaf(yv[c][i], yv[c][i], ss);
+    }
+  }
+  const float total = block_sum<4>(ss, scratch);
+  const float inv = 1.0f / sqrtf(total / (float)hidden + eps);
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const int v4 = threadIdx.x + 256 * c;
+    if (v4 >= nvec) break;
+    float r[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) r[i] = rv[c][i] + scale * (yv[c][i] * inv * wv[c][i]);
+    reinterpret_cast<float4*>(residual + base)[v4] = make_float4(r[0], r[1], r[2], r[3]);
+    if (next) {
+      if (sizeof(T) == 4) {
+        reinterpret_cast<float4*>((float*)next + base)[v4] = make_float4(r[0], r[1], r[2], r[3]);
+      } else {
+        bf16_t h[4] = {__float2bfloat16(r[0]), __float2bfloat16(r[1]), __float2bfloat16(r[2]), __float2bfloat16(r[3])};
+        reinterpret_cast<uint2*>((bf16_t*)next + base)[v4] = *reinterpret_cast<const uint2*>(h);
+      }
+    }
+  }
+}
+
 extern "C" int pae_norm_scale_add(int dtype, float* residual, const void* y, int parts, int64_t part_stride,
                                   const void* weight, int w_is_f32, float eps, float scale, void* next, int num_rows,
                                   int hidden, hipStream_t stream) {
@@ -69,6 +131,15 @@ extern "C" int pae_norm_scale_add(int dtype, float* residual, const void* y, int
               hidden, parts);
   if (num_rows == 0) return 0;
   const size_t lds = hidden <= 8192 ? (size_t)hidden * sizeof(float) : 0;
+  if (hidden % 4 == 0 && hidden <= 4096 && part_stride % 4 == 0 && (dtype == PAE_F32 || dtype == PAE_BF16)) {
+    if (dtype == PAE_F32)
+      norm_scale_add_vec_kernel<float><<<num_rows, 256, 0, stream>>>(residual, y, parts, part_stride, weight, w_is_f32,
+                                                                     eps, scale, (float*)next, hidden);
+    else
+      norm_scale_add_vec_kernel<bf16_t><<<num_rows, 256, 0, stream>>>(residual, y, parts, part_stride, weight, w_is_f32,
+                                                                      eps, scale, (bf16_t*)next, hidden);
+    return pae_check_launch("norm_scale_add");
+  }
   if (dtype == PAE_F32)
     norm_scale_add_kernel<float><<<num_rows, 256, lds, stream>>>(residual, y, parts, part_stride, weight, w_is_f32, eps,
                                                                  scale, (float*)next, hidden);

@@ -28,21 +28,36 @@ __device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z));
 __device__ __forceinline__ float softplus_f(float z) { return z > 20.f ? z : log1pf(expf(z)); }
 
 // seq_runs[s] = (first flat row, rows in this step, tokens held before the step, unused)
+// One workgroup of 128 threads per (token, segment): segments 0 .. G-1 are the q heads, G .. 2G-1 the
+// k heads, 2G .. 2G+H-1 the v heads; the workgroup of segment 0 also computes the token's beta and decay.
 template <typename T>
-__global__ __launch_bounds__(256) void delta_prepare_kernel(
+__global__ __launch_bounds__(128) void delta_prepare_kernel(
     const T* __restrict__ proj, int64_t row_stride, const int* __restrict__ tok_seq, const int* __restrict__ positions,
     const int4* __restrict__ seq_runs, const int* __restrict__ slots, const float* __restrict__ conv_w,
     const float* __restrict__ conv_tail, int64_t tail_slot_stride, int taps, int G, int H, int D, int V,
     const float* __restrict__ a_log, const float* __restrict__ dt_bias, float unit_eps, float* __restrict__ q_out,
     float* __restrict__ k_out, float* __restrict__ v_out, float* __restrict__ beta_out, float* __restrict__ decay_out) {
-  extern __shared__ float chan[];  // [C] the token's convolved, activated channels
-  const int t = blockIdx.x;
+  __shared__ float scratch[2];
+  const int t = blockIdx.x, seg = blockIdx.y;
   const int s = tok_seq[t];
   const int4 run = seq_runs[s];
   const int in_step = t - run.x;  // rows of this sequence before this one in the step
   const int C = 2 * G * D + H * V;
   const float* tail = conv_tail + (int64_t)slots[s] * tail_slot_stride;  // [taps - 1][C], oldest first
-  for (int c = threadIdx.x; c < C; c += 256) {
+  const bool is_v = seg >= 2 * G;
+  const int width = is_v ? V : D;
+  const int c0 = is_v ? 2 * G * D + (seg - 2 * G) * V : seg * D;  // the segment's first channel
+  float* dst = is_v ? v_out + ((int64_t)t * H + seg - 2 * G) * V
+                    : (seg < G ? q_out + ((int64_t)t * G + seg) * D : k_out + ((int64_t)t * G + seg - G) * D);
+  // channels i, i + 128, ... of the segment: convolved and activated; up to 8 a thread are kept (widths to 1,024)
+  float mine[8];
+  float ss = 0.f;
+#pragma unroll
+  for (int n = 0; n < 8; ++n) {
+    const int i = threadIdx.x + 128 * n;
+    mine[n] = 0.f;
+    if (i >= width) break;
+    const int c = c0 + i;
     float sum = 0.f;
     for (int j = 0; j < taps; ++j) {
       const int back = taps - 1 - j;  // tap j weighs the input `back` tokens ago
@@ -51,27 +66,28 @@ __global__ __launch_bounds__(256) void delta_prepare_kernel(
       else x = tail[(int64_t)(taps - 1 - (back - in_step)) * C + c];
       sum = fmaf(conv_w[(int64_t)c * taps + j], x, sum);
     }
-    chan[c] = silu_f(sum);
+    mine[n] = silu_f(sum);
+    ss = fmaf(mine[n], mine[n], ss);
   }
-  __syncthreads();
-  const int wave = threadIdx.x / PAE_WAVE, lane = threadIdx.x % PAE_WAVE;
+  float inv = 1.f;
   const float q_scale = 1.0f / sqrtf((float)D);
-  for (int head = wave; head < 2 * G; head += 4) {  // q heads, then k heads
-    const float* x = chan + head * D;
-    float ss = 0.f;
-    for (int d = lane; d < D; d += PAE_WAVE) ss = fmaf(x[d], x[d], ss);
-    ss = wave_sum(ss);
-    const float inv = 1.0f / sqrtf(ss + unit_eps);
-    const bool is_q = head < G;
-    float* dst = is_q ? q_out + ((int64_t)t * G + head) * D : k_out + ((int64_t)t * G + head - G) * D;
-    for (int d = lane; d < D; d += PAE_WAVE) dst[d] = is_q ? x[d] * inv * q_scale : x[d] * inv;
+  if (!is_v) {  // q and k heads become unit vectors; q is also divided by sqrt(D)
+    ss = block_sum<2>(ss, scratch);
+    inv = 1.0f / sqrtf(ss + unit_eps);
   }
-  for (int i = threadIdx.x; i < H * V; i += 256) v_out[(int64_t)t * H * V + i] = chan[2 * G * D + i];
-  const T* row = proj + (int64_t)t * row_stride;
-  for (int h = threadIdx.x; h < H; h += 256) {
-    const float b = to_f32(row[C + H * V + h]), a = to_f32(row[C + H * V + H + h]);
-    beta_out[(int64_t)t * H + h] = 1.0f / (1.0f + expf(-b));
-    decay_out[(int64_t)t * H + h] = expf(-expf(a_log[h]) * softplus_f(a + dt_bias[h]));
+#pragma unroll
+  for (int n = 0; n < 8; ++n) {
+    const int i = threadIdx.x + 128 * n;
+    if (i >= width) break;
+    dst[i] = is_v ? mine[n] : (seg < G ? mine[n] * inv * q_scale : mine[n] * inv);
+  }
+  if (seg == 0) {
+    const T* row = proj + (int64_t)t * row_stride;
+    for (int h = threadIdx.x; h < H; h += 128) {
+      const float b = to_f32(row[C + H * V + h]), a = to_f32(row[C + H * V + H + h]);
+      beta_out[(int64_t)t * H + h] = 1.0f / (1.0f + expf(-b));
+      decay_out[(int64_t)t * H + h] = expf(-expf(a_log[h]) * softplus_f(a + dt_bias[h]));
+    }
   }
 }
 
@@ -148,6 +164,149 @@ __global__ __launch_bounds__(256) void delta_recurrence_kernel(
   }
 }
 
+// The same recurrence for key widths up to 256, where the chain of dependent steps sets the time: a
+// column is owned by a quad of lanes (sums over the quad are two cross-lane moves inside the
+// register file, no trip through LDS), a lane holds R = D / 4 rows of it (rows 16 i + 4 sub .. + 3, so
+// that the quad's reads of k and q are 64 contiguous bytes).  A workgroup is one wavefront with 16
+// columns: the keys and queries of a step are read from LDS once per wavefront, and with one
+// wavefront a compute unit that traffic stays under the arithmetic (four wavefronts sharing a unit's
+// LDS were bound by it).  The step's inputs reach LDS in chunks of CH tokens: the wavefront fetches
+// the next chunk from memory into registers while it works through the current one, so no step
+// waits for memory.
+__device__ __forceinline__ float quad_sum(float v) {
+  v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xF, 0xF, true));  // lanes (1, 0, 3, 2)
+  v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xF, 0xF, true));  // lanes (2, 3, 0, 1)
+  return v;
+}
+
+template <int R, int CH>
+__global__ __launch_bounds__(PAE_WAVE) void delta_recurrence_quad_kernel(
+    const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v, const float* __restrict__ beta,
+    const float* __restrict__ decay, const int4* __restrict__ seq_runs, const int* __restrict__ slots,
+    float* __restrict__ state, int64_t state_slot_stride, int G, int H, int D, int V, float* __restrict__ out) {
+  constexpr int DP = 4 * R;                // rows of a column, padded
+  constexpr int KQ = CH * DP / PAE_WAVE;   // numbers of k (and of q) a lane fetches per chunk
+  constexpr int VN = CH * 16 / PAE_WAVE;   // of v
+  static_assert(CH * DP % (4 * PAE_WAVE) == 0 && CH * 16 % PAE_WAVE == 0 && 2 * CH <= PAE_WAVE, "chunk shape");
+  __shared__ __attribute__((aligned(16))) float s_k[CH * DP];
+  __shared__ __attribute__((aligned(16))) float s_q[CH * DP];
+  __shared__ float s_v[CH * 16];
+  __shared__ float s_bd[2 * CH];           // beta, then decay
+  const int s = blockIdx.z, h = blockIdx.y, col0 = blockIdx.x * 16;
+  const int lane = threadIdx.x;
+  const int col = col0 + lane / 4, sub = lane % 4;
+  const bool live = col < V;
+  const int4 run = seq_runs[s];
+  const int g = h / (H / G);
+  float* column = state + (int64_t)slots[s] * state_slot_stride + ((int64_t)h * V + (live ? col : 0)) * D;
+  float S[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int d = (r >> 2) * 16 + sub * 4 + (r & 3);
+    S[r] = (live && d < D) ? column[d] : 0.f;
+  }
+  const bool vec = D % 4 == 0;
+  float pk[KQ], pq[KQ], pv[VN], pbd;
+  // a lane's share of the chunk that starts at token `first` of the run, from memory into registers
+  auto fetch = [&](int first) {
+    if (vec) {
+#pragma unroll
+      for (int p = 0; p < KQ / 4; ++p) {
+        const int e = (lane + PAE_WAVE * p) * 4, i = e / DP, d = e % DP;
+        float4 a = make_float4(0.f, 0.f, 0.f, 0.f), b = a;
+        if (first + i < run.y && d < D) {
+          const int64_t at = ((int64_t)(run.x + first + i) * G + g) * D + d;
+          a = *reinterpret_cast<const float4*>(k + at);
+          b = *reinterpret_cast<const float4*>(q + at);
+        }
+        pk[4 * p] = a.x; pk[4 * p + 1] = a.y; pk[4 * p + 2] = a.z; pk[4 * p + 3] = a.w;
+        pq[4 * p] = b.x; pq[4 * p + 1] = b.y; pq[4 * p + 2] = b.z; pq[4 * p + 3] = b.w;
+      }
+    } else {
+#pragma unroll
+      for (int p = 0; p < KQ; ++p) {
+        const int e = lane + PAE_WAVE * p, i = e / DP, d = e % DP;
+        const bool there = first + i < run.y && d < D;
+        const int64_t at = ((int64_t)(run.x + first + i) * G + g) * D + d;
+        pk[p] = there ? k[at] : 0.f;
+        pq[p] = there ? q[at] : 0.f;
+      }
+    }
+#pragma unroll
+    for (int p = 0; p < VN; ++p) {
+      const int e = lane + PAE_WAVE * p, i = e / 16, c = col0 + e % 16;
+      pv[p] = (first + i < run.y && c < V) ? v[((int64_t)(run.x + first + i) * H + h) * V + c] : 0.f;
+    }
+    pbd = 0.f;
+    if (lane < 2 * CH && first + lane % CH < run.y)
+      pbd = (lane < CH ? beta : decay)[(int64_t)(run.x + first + lane % CH) * H + h];
+  };
+  auto stage = [&]() {
+    if (vec) {
+#pragma unroll
+      for (int p = 0; p < KQ / 4; ++p) {
+        const int e = (lane + PAE_WAVE * p) * 4;
+        *reinterpret_cast<float4*>(s_k + e) = make_float4(pk[4 * p], pk[4 * p + 1], pk[4 * p + 2], pk[4 * p + 3]);
+        *reinterpret_cast<float4*>(s_q + e) = make_float4(pq[4 * p], pq[4 * p + 1], pq[4 * p + 2], pq[4 * p + 3]);
+      }
+    } else {
+#pragma unroll
+      for (int p = 0; p < KQ; ++p) {
+        s_k[lane + PAE_WAVE * p] = pk[p];
+        s_q[lane + PAE_WAVE * p] = pq[p];
+      }
+    }
+#pragma unroll
+    for (int p = 0; p < VN; ++p) s_v[lane + PAE_WAVE * p] = pv[p];
+    if (lane < 2 * CH) s_bd[lane] = pbd;
+  };
+  fetch(0);
+  for (int first = 0; first < run.y; first += CH) {
+    __syncthreads();  // the chunk before has been worked through
+    stage();
+    __syncthreads();
+    if (first + CH < run.y) fetch(first + CH);
+    const int n = min(CH, run.y - first);
+    for (int i = 0; i < n; ++i) {
+      const float* kt = s_k + i * DP;
+      const float* qt = s_q + i * DP;
+      const float dec = s_bd[CH + i], b = s_bd[i], vt = s_v[i * 16 + lane / 4];
+      float kr[R];
+      float dot = 0.f;
+#pragma unroll
+      for (int r4 = 0; r4 < R / 4; ++r4) {
+        const float4 k4 = *reinterpret_cast<const float4*>(kt + r4 * 16 + sub * 4);
+        kr[4 * r4] = k4.x; kr[4 * r4 + 1] = k4.y; kr[4 * r4 + 2] = k4.z; kr[4 * r4 + 3] = k4.w;
+      }
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        S[r] = dec * S[r];
+        dot = fmaf(S[r], kr[r], dot);
+      }
+      dot = quad_sum(dot);
+      const float u = b * (vt - dot);
+      float o = 0.f;
+#pragma unroll
+      for (int r4 = 0; r4 < R / 4; ++r4) {
+        const float4 q4 = *reinterpret_cast<const float4*>(qt + r4 * 16 + sub * 4);
+        S[4 * r4 + 0] = fmaf(kr[4 * r4 + 0], u, S[4 * r4 + 0]); o = fmaf(S[4 * r4 + 0], q4.x, o);
+        S[4 * r4 + 1] = fmaf(kr[4 * r4 + 1], u, S[4 * r4 + 1]); o = fmaf(S[4 * r4 + 1], q4.y, o);
+        S[4 * r4 + 2] = fmaf(kr[4 * r4 + 2], u, S[4 * r4 + 2]); o = fmaf(S[4 * r4 + 2], q4.z, o);
+        S[4 * r4 + 3] = fmaf(kr[4 * r4 + 3], u, S[4 * r4 + 3]); o = fmaf(S[4 * r4 + 3], q4.w, o);
+      }
+      o = quad_sum(o);
+      if (live && sub == 0) out[((int64_t)(run.x + first + i) * H + h) * V + col] = o;
+    }
+  }
+  if (live) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int d = (r >> 2) * 16 + sub * 4 + (r & 3);
+      if (d < D) column[d] = S[r];
+    }
+  }
+}
+
 template <typename T>
 __global__ __launch_bounds__(PAE_WAVE) void delta_gated_norm_kernel(const float* __restrict__ o, const T* __restrict__ proj,
                                                                     int64_t row_stride, int gate_offset,
@@ -163,6 +322,30 @@ __global__ __launch_bounds__(PAE_WAVE) void delta_gated_norm_kernel(const float*
   const T* gate = proj + t * row_stride + gate_offset + h * V;
   for (int i = lane; i < V; i += PAE_WAVE)
     out[(t * H + h) * V + i] = from_f32<T>(x[i] * inv * load_param(weight, w_is_f32, i) * silu_f(to_f32(gate[i])));
+}
+
+static int lanes_per_column(int D, int R);
+
+static void launch_recurrence(const float* q, const float* k, const float* v, const float* beta, const float* decay,
+                              const int4* runs, const int* slots, float* state, int64_t state_slot_stride, int G, int H,
+                              int D, int V, int num_seqs, float* o, hipStream_t stream) {
+  dim3 quad_grid((V + 15) / 16, H, num_seqs);
+  // (tokens a chunk: fewer with wider keys, so that the registers that hold the next chunk stay few)
+#define QUAD(R, CH)                                                                                      \
+  delta_recurrence_quad_kernel<R, CH><<<quad_grid, PAE_WAVE, 0, stream>>>(q, k, v, beta, decay, runs, slots, state, \
+                                                                          state_slot_stride, G, H, D, V, o)
+  if (D <= 16) QUAD(4, 32);
+  else if (D <= 32) QUAD(8, 32);
+  else if (D <= 64) QUAD(16, 16);
+  else if (D <= 128) QUAD(32, 8);
+  else if (D <= 256) QUAD(64, 4);
+  else {
+    const int L = lanes_per_column(D, 16);
+    dim3 rec_grid((V + 256 / L - 1) / (256 / L), H, num_seqs);
+    delta_recurrence_kernel<16><<<rec_grid, 256, 0, stream>>>(q, k, v, beta, decay, runs, slots, state,
+                                                              state_slot_stride, G, H, D, V, L, o);
+  }
+#undef QUAD
 }
 
 static int lanes_per_column(int D, int R) {
@@ -182,7 +365,7 @@ extern "C" int pae_delta_rule_step(int dtype, const void* proj, int64_t row_stri
   PAE_REQUIRE(D <= 1024, "delta rule: key width %d exceeds 1024", D);
   PAE_REQUIRE(H <= 65535 && num_seqs <= 65535, "delta rule: %d heads, %d sequences exceed the grid", H, num_seqs);
   const int64_t C = 2 * (int64_t)G * D + (int64_t)H * V;
-  PAE_REQUIRE(C * 4 <= 64 * 1024, "delta rule: %lld convolved channels exceed the kernel's 64 KB of LDS", (long long)C);
+  PAE_REQUIRE(V <= 1024 && 2 * G + H <= 65535, "delta rule: value width %d or %d heads exceed the kernels' limits", V, 2 * G + H);
   PAE_REQUIRE(row_stride >= C + (int64_t)H * V + 2 * H, "delta rule: row stride %lld too small", (long long)row_stride);
   PAE_REQUIRE(dtype == PAE_F32 || dtype == PAE_BF16, "delta rule: unknown dtype code %d", dtype);
   if (num_tokens <= 0 || num_seqs <= 0) return 0;
@@ -194,20 +377,16 @@ extern "C" int pae_delta_rule_step(int dtype, const void* proj, int64_t row_stri
   float* decay = beta + (int64_t)num_tokens * H;
   float* o = decay + (int64_t)num_tokens * H;
   const int4* runs = (const int4*)seq_runs;
-  const int R = 16;
-  const int L = lanes_per_column(D, R);
   dim3 tail_grid((unsigned)((C + 255) / 256), num_seqs);
-  dim3 rec_grid((V + 256 / L - 1) / (256 / L), H, num_seqs);
   dim3 norm_grid(num_tokens, H);
 #define DELTA_LAUNCH(T)                                                                                                 \
-  delta_prepare_kernel<T><<<num_tokens, 256, (size_t)C * 4, stream>>>(                                                  \
+  delta_prepare_kernel<T><<<dim3(num_tokens, 2 * G + H), 128, 0, stream>>>(                                             \
       (const T*)proj, row_stride, tok_seq, positions, runs, slots, conv_w, conv_tail, tail_slot_stride, taps, G, H, D,  \
       V, a_log, dt_bias, unit_eps, q, k, v, beta, decay);                                                               \
   if (taps > 1)                                                                                                         \
     delta_conv_tail_kernel<T><<<tail_grid, 256, 0, stream>>>((const T*)proj, row_stride, runs, slots, conv_tail,        \
                                                              tail_slot_stride, taps, (int)C);                           \
-  delta_recurrence_kernel<16><<<rec_grid, 256, 0, stream>>>(q, k, v, beta, decay, runs, slots, state,                   \
-                                                            state_slot_stride, G, H, D, V, L, o);                       \
+  launch_recurrence(q, k, v, beta, decay, runs, slots, state, state_slot_stride, G, H, D, V, num_seqs, o, stream);      \
   delta_gated_norm_kernel<T><<<norm_grid, PAE_WAVE, 0, stream>>>(o, (const T*)proj, row_stride, (int)C, norm_w,         \
                                                                  w_is_f32, norm_eps, H, V, (T*)out)
   if (dtype == PAE_F32) {

@@ -49,8 +49,8 @@ class GatedDeltaMixer(Part):
             raise ValueError(f"key_dim {spec.key_dim}: the recurrence kernel takes up to 1024")
         if not 1 <= spec.conv_taps <= 64:
             raise ValueError(f"conv_taps {spec.conv_taps} is outside 1..64")
-        if self.channels * 4 > 64 * 1024:
-            raise ValueError(f"{self.channels} convolved channels exceed what the kernel holds in LDS (16,384)")
+        if not 0 < spec.value_dim <= 1024:
+            raise ValueError(f"value_dim {spec.value_dim}: the kernels take up to 1024")
 
     @property
     def channels(self) -> int:
