@@ -164,37 +164,40 @@ __global__ __launch_bounds__(256) void delta_recurrence_kernel(
   }
 }
 
-// The same recurrence for key widths up to 256, where the chain of dependent steps sets the time: a
-// column is owned by a quad of lanes (sums over the quad are two cross-lane moves inside the
-// register file, no trip through LDS), a lane holds R = D / 4 rows of it (rows 16 i + 4 sub .. + 3, so
-// that the quad's reads of k and q are 64 contiguous bytes).  A workgroup is one wavefront with 16
-// columns: the keys and queries of a step are read from LDS once per wavefront, and with one
-// wavefront a compute unit that traffic stays under the arithmetic (four wavefronts sharing a unit's
-// LDS were bound by it).  The step's inputs reach LDS in chunks of CH tokens: the wavefront fetches
-// the next chunk from memory into registers while it works through the current one, so no step
-// waits for memory.
-__device__ __forceinline__ float quad_sum(float v) {
-  v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xF, 0xF, true));  // lanes (1, 0, 3, 2)
+// The same recurrence for key widths up to 256, where the chain of dependent steps sets the time.  A
+// column is owned by a group of L = 4, 8 or 16 neighbouring lanes, whose sums are added by cross-lane
+// moves inside the register file (no trip through LDS); a lane holds R = D / L rows of its column
+// (rows 4 L i + 4 sub .. + 3, so that a group's reads of k and q are contiguous).  The wider the keys,
+// the more lanes share a column, which keeps the chain of a step short: 4 R multiply-adds and two
+// sums over the group.  A workgroup has 16 columns (16 L threads); the step's inputs reach it
+// through LDS in chunks of CH tokens, the next chunk being fetched from memory into registers while
+// the current one is worked through, so no step waits for memory.
+template <int L>
+__device__ __forceinline__ float group_sum(float v) {
+  v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xF, 0xF, true));  // lanes (1, 0, 3, 2) of a quad
   v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xF, 0xF, true));  // lanes (2, 3, 0, 1)
+  if (L >= 8) v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x141, 0xF, 0xF, true));   // 8 lanes mirrored
+  if (L >= 16) v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x140, 0xF, 0xF, true));  // 16 lanes mirrored
   return v;
 }
 
-template <int R, int CH>
-__global__ __launch_bounds__(PAE_WAVE) void delta_recurrence_quad_kernel(
+template <int R, int L, int CH>
+__global__ __launch_bounds__(16 * L) void delta_recurrence_group_kernel(
     const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v, const float* __restrict__ beta,
     const float* __restrict__ decay, const int4* __restrict__ seq_runs, const int* __restrict__ slots,
     float* __restrict__ state, int64_t state_slot_stride, int G, int H, int D, int V, float* __restrict__ out) {
-  constexpr int DP = 4 * R;                // rows of a column, padded
-  constexpr int KQ = CH * DP / PAE_WAVE;   // numbers of k (and of q) a lane fetches per chunk
-  constexpr int VN = CH * 16 / PAE_WAVE;   // of v
-  static_assert(CH * DP % (4 * PAE_WAVE) == 0 && CH * 16 % PAE_WAVE == 0 && 2 * CH <= PAE_WAVE, "chunk shape");
+  constexpr int NT = 16 * L;         // threads: 16 columns of L lanes
+  constexpr int DP = L * R;          // rows of a column, padded
+  constexpr int KQ = CH * DP / NT;   // numbers of k (and of q) a thread fetches per chunk
+  constexpr int VN = CH * 16 / NT;   // of v
+  static_assert(R % 4 == 0 && CH * DP % (4 * NT) == 0 && CH * 16 % NT == 0 && 2 * CH <= NT, "chunk shape");
   __shared__ __attribute__((aligned(16))) float s_k[CH * DP];
   __shared__ __attribute__((aligned(16))) float s_q[CH * DP];
   __shared__ float s_v[CH * 16];
-  __shared__ float s_bd[2 * CH];           // beta, then decay
+  __shared__ float s_bd[2 * CH];     // beta, then decay
   const int s = blockIdx.z, h = blockIdx.y, col0 = blockIdx.x * 16;
-  const int lane = threadIdx.x;
-  const int col = col0 + lane / 4, sub = lane % 4;
+  const int tid = threadIdx.x;
+  const int col = col0 + tid / L, sub = tid % L;
   const bool live = col < V;
   const int4 run = seq_runs[s];
   const int g = h / (H / G);
@@ -202,17 +205,17 @@ __global__ __launch_bounds__(PAE_WAVE) void delta_recurrence_quad_kernel(
   float S[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    const int d = (r >> 2) * 16 + sub * 4 + (r & 3);
+    const int d = (r >> 2) * (4 * L) + sub * 4 + (r & 3);
     S[r] = (live && d < D) ? column[d] : 0.f;
   }
   const bool vec = D % 4 == 0;
   float pk[KQ], pq[KQ], pv[VN], pbd;
-  // a lane's share of the chunk that starts at token `first` of the run, from memory into registers
+  // a thread's share of the chunk that starts at token `first` of the run, from memory into registers
   auto fetch = [&](int first) {
     if (vec) {
 #pragma unroll
       for (int p = 0; p < KQ / 4; ++p) {
-        const int e = (lane + PAE_WAVE * p) * 4, i = e / DP, d = e % DP;
+        const int e = (tid + NT * p) * 4, i = e / DP, d = e % DP;
         float4 a = make_float4(0.f, 0.f, 0.f, 0.f), b = a;
         if (first + i < run.y && d < D) {
           const int64_t at = ((int64_t)(run.x + first + i) * G + g) * D + d;
@@ -225,7 +228,7 @@ __global__ __launch_bounds__(PAE_WAVE) void delta_recurrence_quad_kernel(
     } else {
 #pragma unroll
       for (int p = 0; p < KQ; ++p) {
-        const int e = lane + PAE_WAVE * p, i = e / DP, d = e % DP;
+        const int e = tid + NT * p, i = e / DP, d = e % DP;
         const bool there = first + i < run.y && d < D;
         const int64_t at = ((int64_t)(run.x + first + i) * G + g) * D + d;
         pk[p] = there ? k[at] : 0.f;
@@ -234,31 +237,31 @@ __global__ __launch_bounds__(PAE_WAVE) void delta_recurrence_quad_kernel(
     }
 #pragma unroll
     for (int p = 0; p < VN; ++p) {
-      const int e = lane + PAE_WAVE * p, i = e / 16, c = col0 + e % 16;
+      const int e = tid + NT * p, i = e / 16, c = col0 + e % 16;
       pv[p] = (first + i < run.y && c < V) ? v[((int64_t)(run.x + first + i) * H + h) * V + c] : 0.f;
     }
     pbd = 0.f;
-    if (lane < 2 * CH && first + lane % CH < run.y)
-      pbd = (lane < CH ? beta : decay)[(int64_t)(run.x + first + lane % CH) * H + h];
+    if (tid < 2 * CH && first + tid % CH < run.y)
+      pbd = (tid < CH ? beta : decay)[(int64_t)(run.x + first + tid % CH) * H + h];
   };
   auto stage = [&]() {
     if (vec) {
 #pragma unroll
       for (int p = 0; p < KQ / 4; ++p) {
-        const int e = (lane + PAE_WAVE * p) * 4;
+        const int e = (tid + NT * p) * 4;
         *reinterpret_cast<float4*>(s_k + e) = make_float4(pk[4 * p], pk[4 * p + 1], pk[4 * p + 2], pk[4 * p + 3]);
         *reinterpret_cast<float4*>(s_q + e) = make_float4(pq[4 * p], pq[4 * p + 1], pq[4 * p + 2], pq[4 * p + 3]);
       }
     } else {
 #pragma unroll
       for (int p = 0; p < KQ; ++p) {
-        s_k[lane + PAE_WAVE * p] = pk[p];
-        s_q[lane + PAE_WAVE * p] = pq[p];
+        s_k[tid + NT * p] = pk[p];
+        s_q[tid + NT * p] = pq[p];
       }
     }
 #pragma unroll
-    for (int p = 0; p < VN; ++p) s_v[lane + PAE_WAVE * p] = pv[p];
-    if (lane < 2 * CH) s_bd[lane] = pbd;
+    for (int p = 0; p < VN; ++p) s_v[tid + NT * p] = pv[p];
+    if (tid < 2 * CH) s_bd[tid] = pbd;
   };
   fetch(0);
   for (int first = 0; first < run.y; first += CH) {
@@ -270,12 +273,12 @@ __global__ __launch_bounds__(PAE_WAVE) void delta_recurrence_quad_kernel(
     for (int i = 0; i < n; ++i) {
       const float* kt = s_k + i * DP;
       const float* qt = s_q + i * DP;
-      const float dec = s_bd[CH + i], b = s_bd[i], vt = s_v[i * 16 + lane / 4];
+      const float dec = s_bd[CH + i], b = s_bd[i], vt = s_v[i * 16 + tid / L];
       float kr[R];
       float dot = 0.f;
 #pragma unroll
       for (int r4 = 0; r4 < R / 4; ++r4) {
-        const float4 k4 = *reinterpret_cast<const float4*>(kt + r4 * 16 + sub * 4);
+        const float4 k4 = *reinterpret_cast<const float4*>(kt + r4 * (4 * L) + sub * 4);
         kr[4 * r4] = k4.x; kr[4 * r4 + 1] = k4.y; kr[4 * r4 + 2] = k4.z; kr[4 * r4 + 3] = k4.w;
       }
 #pragma unroll
@@ -283,25 +286,25 @@ __global__ __launch_bounds__(PAE_WAVE) void delta_recurrence_quad_kernel(
         S[r] = dec * S[r];
         dot = fmaf(S[r], kr[r], dot);
       }
-      dot = quad_sum(dot);
+      dot = group_sum<L>(dot);
       const float u = b * (vt - dot);
       float o = 0.f;
 #pragma unroll
       for (int r4 = 0; r4 < R / 4; ++r4) {
-        const float4 q4 = *reinterpret_cast<const float4*>(qt + r4 * 16 + sub * 4);
+        const float4 q4 = *reinterpret_cast<const float4*>(qt + r4 * (4 * L) + sub * 4);
         S[4 * r4 + 0] = fmaf(kr[4 * r4 + 0], u, S[4 * r4 + 0]); o = fmaf(S[4 * r4 + 0], q4.x, o);
         S[4 * r4 + 1] = fmaf(kr[4 * r4 + 1], u, S[4 * r4 + 1]); o = fmaf(S[4 * r4 + 1], q4.y, o);
         S[4 * r4 + 2] = fmaf(kr[4 * r4 + 2], u, S[4 * r4 + 2]); o = fmaf(S[4 * r4 + 2], q4.z, o);
         S[4 * r4 + 3] = fmaf(kr[4 * r4 + 3], u, S[4 * r4 + 3]); o = fmaf(S[4 * r4 + 3], q4.w, o);
       }
-      o = quad_sum(o);
+      o = group_sum<L>(o);
       if (live && sub == 0) out[((int64_t)(run.x + first + i) * H + h) * V + col] = o;
     }
   }
   if (live) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      const int d = (r >> 2) * 16 + sub * 4 + (r & 3);
+      const int d = (r >> 2) * (4 * L) + sub * 4 + (r & 3);
       if (d < D) column[d] = S[r];
     }
   }
@@ -329,23 +332,23 @@ static int lanes_per_column(int D, int R);
 static void launch_recurrence(const float* q, const float* k, const float* v, const float* beta, const float* decay,
                               const int4* runs, const int* slots, float* state, int64_t state_slot_stride, int G, int H,
                               int D, int V, int num_seqs, float* o, hipStream_t stream) {
-  dim3 quad_grid((V + 15) / 16, H, num_seqs);
-  // (tokens a chunk: fewer with wider keys, so that the registers that hold the next chunk stay few)
-#define QUAD(R, CH)                                                                                      \
-  delta_recurrence_quad_kernel<R, CH><<<quad_grid, PAE_WAVE, 0, stream>>>(q, k, v, beta, decay, runs, slots, state, \
-                                                                          state_slot_stride, G, H, D, V, o)
-  if (D <= 16) QUAD(4, 32);
-  else if (D <= 32) QUAD(8, 32);
-  else if (D <= 64) QUAD(16, 16);
-  else if (D <= 128) QUAD(32, 8);
-  else if (D <= 256) QUAD(64, 4);
+  dim3 group_grid((V + 15) / 16, H, num_seqs);
+  // (rows a lane, lanes a column, tokens a chunk)
+#define GROUP(R, L, CH)                                                                                          \
+  delta_recurrence_group_kernel<R, L, CH><<<group_grid, 16 * L, 0, stream>>>(q, k, v, beta, decay, runs, slots, state, \
+                                                                             state_slot_stride, G, H, D, V, o)
+  if (D <= 16) GROUP(4, 4, 32);
+  else if (D <= 32) GROUP(8, 4, 32);
+  else if (D <= 64) GROUP(8, 8, 16);
+  else if (D <= 128) GROUP(8, 16, 16);
+  else if (D <= 256) GROUP(16, 16, 16);
   else {
     const int L = lanes_per_column(D, 16);
     dim3 rec_grid((V + 256 / L - 1) / (256 / L), H, num_seqs);
     delta_recurrence_kernel<16><<<rec_grid, 256, 0, stream>>>(q, k, v, beta, decay, runs, slots, state,
                                                               state_slot_stride, G, H, D, V, L, o);
   }
-#undef QUAD
+#undef GROUP
 }
 
 static int lanes_per_column(int D, int R) {
