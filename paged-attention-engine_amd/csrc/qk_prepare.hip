@@ -25,6 +25,15 @@ __global__ __launch_bounds__(256) void qk_norm_rotate_store_kernel(
   const int t = blockIdx.x;
   T* row = qkv + (int64_t)t * row_stride;
   const int nq = nh * hd, nk = nkv * hd;
+  // the token's place in the cache is asked for first: the answer arrives while the sums are formed
+  const int pos = positions[t];
+  const int off = pos % bs;
+  int64_t k_base = 0, v_base = 0;  // element offsets of (block, kv head 0) in the pools
+  if (write_kv) {
+    const int64_t block = block_tables[(int64_t)tok_seq[t] * max_blocks + pos / bs];
+    k_base = block * nkv * (int64_t)bs * hd;
+    v_base = block * nkv * (int64_t)bs * vd;
+  }
   float inv_q = 1.f, inv_k = 1.f;
   if (q_w) {
     float sq = 0.f, sk = 0.f;
@@ -36,14 +45,6 @@ __global__ __launch_bounds__(256) void qk_norm_rotate_store_kernel(
       sk = block_sum<4>(sk, scratch);
       inv_k = 1.0f / sqrtf(sk / (float)nk + eps);
     }
-  }
-  const int pos = positions[t];
-  const int off = pos % bs;
-  int64_t k_base = 0, v_base = 0;  // element offsets of (block, kv head 0) in the pools
-  if (write_kv) {
-    const int64_t block = block_tables[(int64_t)tok_seq[t] * max_blocks + pos / bs];
-    k_base = block * nkv * (int64_t)bs * hd;
-    v_base = block * nkv * (int64_t)bs * vd;
   }
   // feature j of the row (j < nq + nk), normalised
   auto at = [&](int j) {
