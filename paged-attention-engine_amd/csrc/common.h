@@ -45,6 +45,13 @@ __device__ __forceinline__ float load_param(const void* p, int is_f32, int64_t i
   return is_f32 ? ((const float*)p)[i] : __bfloat162float(((const bf16_t*)p)[i]);
 }
 
+// Activations by code (0 gelu by erf, 1 gelu by tanh, 2 silu), in float32.
+__device__ __forceinline__ float act_of(float z, int kind) {
+  if (kind == 0) return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f));
+  if (kind == 1) return 0.5f * z * (1.0f + tanhf(0.79788456080286536f * (z + 0.044715f * z * z * z)));
+  return z / (1.0f + expf(-z));
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int off = PAE_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, PAE_WAVE);

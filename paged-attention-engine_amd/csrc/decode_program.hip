@@ -708,7 +708,7 @@ extern "C" int pae_program_put_product(void* phases, int index, int epilogue, vo
   ph.M = M; ph.N = N; ph.K = K; ph.splits = splits; ph.k_per_split = k_per_split; ph.b_is_f32 = b_is_f32;
   ph.W = (const bf16_t*)W; ph.bias = bias; ph.A = (const bf16_t*)A; ph.out = out;
   ph.lda = lda; ph.ldc = ldc;
-  ph.norm = SkinnyNorm{row_stats, row_stat_tiles, row_eps, (bf16_t*)next_rows, ld_next, next_w, next_w_is_f32, next_stats};
+  ph.norm = SkinnyNorm{row_stats, row_stat_tiles, row_eps, (bf16_t*)next_rows, ld_next, next_w, next_w_is_f32, 0, next_stats};
   if (rope) ph.rope = *rope;
   ph.ticket_parts = ticketed ? ticket_parts : nullptr;
   ph.ticket_counters = ticketed ? ticket_counters : nullptr;

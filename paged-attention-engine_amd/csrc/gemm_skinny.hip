@@ -562,8 +562,19 @@ extern "C" int pae_gemm_skinny(int epilogue, void* out, int64_t ldc, const void*
                                int64_t ld_next, const void* next_w, int next_w_is_f32, float* next_stats,
                                hipStream_t stream) {
   PAE_REQUIRE(epilogue != EPI_ROPE, "gemm_skinny: the rotating epilogue has an entry point of its own");
-  const SkinnyNorm norm{row_stats, row_stat_tiles, row_eps, (bf16_t*)next_rows, ld_next, next_w, next_w_is_f32, next_stats};
+  const SkinnyNorm norm{row_stats, row_stat_tiles, row_eps, (bf16_t*)next_rows, ld_next, next_w, next_w_is_f32, 0, next_stats};
   return launch_skinny(epilogue, out, ldc, A, lda, W, bias, b_is_f32, M, N, K, splits, part_stride, SkinnyRope{},
+                       SkinnyTickets{ticket_parts, ticket_counters}, norm, stream);
+}
+
+// out[M, N] = bfloat16(act(A W^T + bias)): the plain epilogue with an activation (0 gelu by erf, 1 gelu by tanh,
+// 2 silu) on the finished sums, in float32, before they are rounded.
+extern "C" int pae_gemm_skinny_act(void* out, int64_t ldc, const void* A, int64_t lda, const void* W, const void* bias,
+                                   int b_is_f32, int M, int N, int K, int splits, float* ticket_parts,
+                                   int* ticket_counters, int act, hipStream_t stream) {
+  PAE_REQUIRE(act >= 0 && act <= 2, "gemm_skinny_act: unknown activation %d", act);
+  const SkinnyNorm norm{nullptr, 0, 0.f, nullptr, 0, nullptr, 0, act + 1, nullptr};
+  return launch_skinny(EPI_BF16, out, ldc, A, lda, W, bias, b_is_f32, M, N, K, splits, 0, SkinnyRope{},
                        SkinnyTickets{ticket_parts, ticket_counters}, norm, stream);
 }
 
@@ -595,7 +606,7 @@ extern "C" int pae_gemm_skinny_rope(void* q_out, int64_t ldq, const void* A, int
               "gemm_skinny_rope: the cache write needs tables and pools");
   SkinnyRope rope{cos_sin, positions, tok_seq, block_tables, (bf16_t*)k_cache, (bf16_t*)v_cache,
                   nh, nkv, hd, rot, max_blocks, bs};
-  const SkinnyNorm norm{row_stats, row_stat_tiles, row_eps, nullptr, 0, nullptr, 0, nullptr};
+  const SkinnyNorm norm{row_stats, row_stat_tiles, row_eps, nullptr, 0, nullptr, 0, 0, nullptr};
   return launch_skinny(EPI_ROPE, q_out, ldq, A, lda, W, bias, b_is_f32, M, (nh + 2 * nkv) * hd, K, splits, 0, rope,
                        SkinnyTickets{ticket_parts, ticket_counters}, norm, stream);
 }

@@ -34,6 +34,7 @@ struct SkinnyNorm {
   int64_t ld_next;
   const void* next_w;      // [N] weight of the norm that follows
   int next_w_is_f32;
+  int act;                 // EPI_BF16: 0, or 1 + the code of an activation (see act_of) that the sums pass before they are rounded
   float* next_stats;       // [M][(N + 15) / 16]
 };
 
@@ -172,7 +173,7 @@ struct SkinnyRope {
 
 __device__ __forceinline__ SkinnyNorm in_memory(const SkinnyNorm& n) {
   return SkinnyNorm{in_memory(n.row_stats), n.row_stat_tiles, n.eps, in_memory(n.next_rows), n.ld_next,
-                    in_memory(n.next_w), n.next_w_is_f32, in_memory(n.next_stats)};
+                    in_memory(n.next_w), n.next_w_is_f32, n.act, in_memory(n.next_stats)};
 }
 __device__ __forceinline__ SkinnyRope in_memory(const SkinnyRope& r) {
   return SkinnyRope{in_memory(r.cos_sin), in_memory(r.positions), in_memory(r.tok_seq), in_memory(r.block_tables),
@@ -438,6 +439,10 @@ __device__ __forceinline__ void skinny_epilogue(const f32x4 (&acc)[RT][MT], int 
           else
             for (int i = 0; i < 4 && n + i < N; ++i) put<THROUGH>(dst + i, v[i]);
         } else {
+          if (EPI == EPI_BF16 && norm.act) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) v[i] = act_of(v[i], norm.act - 1);
+          }
           bf16_t* dst = (bf16_t*)out + (int64_t)m * ldc + n;
           if (vec && n + 4 <= N) {
             s16x4 p;

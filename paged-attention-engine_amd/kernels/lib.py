@@ -67,6 +67,7 @@ def _declare(lib) -> None:
         "pae_embedding_rows": [I, P, P, P, I, I, I, F, P, P, I, P, P],
         "pae_scaled_rows": [P, P, P, I, F, I, I, P],
         "pae_skinny_ticket_slots": [I, I],
+        "pae_gemm_skinny_act": [P, L, P, L, P, P, I, I, I, I, I, P, P, I, P],
         "pae_gemm_plain": [I, I, P, L, P, L, P, P, I, I, I, I, P],
         "pae_paged_attention_generic": [I, P, L, P, L, P, P, P, P, P, I, I, I, I, I, I, F, I, P],
         "pae_paged_attention_capped": [I, P, L, P, L, P, P, P, P, P, I, I, I, I, I, I, I, F, I, F, P, P],
@@ -662,6 +663,23 @@ def gemm_skinny(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optio
         M * N, _ptr(parts), _ptr(counters), sp, st, se, nr, ld_next, nw, nwf, ns, _stream()))
     if checking:
         _check_ticket_sums(out, before, a, w, bias, epilogue, splits, row_scale, following)
+
+
+def gemm_skinny_act(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, kind: str, splits: int = 1,
+                    bias: Optional[torch.Tensor] = None) -> None:
+    """out [M, N] bfloat16 = act(a @ w^T + bias) for at most 64 rows of `a`: the weight-streaming product
+    with the activation `kind` (see ACTIVATIONS) on its finished float32 sums, rounded once."""
+    _not_while_recording("gemm_skinny_act")
+    _gpu(out, a, w, bias)
+    M, K_ = a.shape
+    N = w.shape[0]
+    assert skinny_supported(a, w) and w.shape == (N, K_) and w.is_contiguous() and out.is_contiguous()
+    assert out.shape == (M, N) and out.dtype == torch.bfloat16 and kind in ACTIVATIONS
+    bp, bf = _param(bias)
+    parts, counters = _ticket_scratch(a.device, M, N, splits)
+    _launch_ticketed(counters, lambda: library().pae_gemm_skinny_act(
+        out.data_ptr(), out.stride(0), a.data_ptr(), a.stride(0), w.data_ptr(), bp, bf, M, N, K_, splits, _ptr(parts),
+        _ptr(counters), ACTIVATIONS[kind], _stream()))
 
 
 # PAE_CHECK_TICKETS=sums: every product whose k ranges are added up inside the kernel is computed a

@@ -96,6 +96,14 @@ class DenseFeedForward(Part):
         self.down = Linear(self.matrix(weights[prefix + s.down_name + s.weight_suffix]))
 
     def forward(self, ctx, x):
-        act = self.up(plain_rows(x))
-        K.activation(act, self.spec.activation)
+        """Up to 64 rows the activation runs in the up product's epilogue, on its float32 sums; above,
+        the platform library's product is followed by the activation kernel."""
+        x = plain_rows(x)
+        if x.shape[0] and K.skinny_supported(x, self.up.weight):
+            act = torch.empty((x.shape[0], self.spec.intermediate_size), dtype=x.dtype, device=x.device)
+            splits = K.whole_sum_splits(self.spec.intermediate_size, self.spec.hidden_size, x.shape[0])
+            K.gemm_skinny_act(act, x, self.up.weight, self.spec.activation, splits)
+        else:
+            act = self.up(x)
+            K.activation(act, self.spec.activation)
         return self.down.branch(act, getattr(ctx, "sink", None))

@@ -62,8 +62,14 @@ S = {"architecture": "Danonex", "vocab": 400, "width": 128, "norm": {"eps": 1e-5
          layer(delta(4, 2, 32, 32, 4)),
          layer(attention(3, 3, 32, 32, 0.5, softcap=None, rot_dims=32, base=100.0, scaling=None), ff=64),
      ]}
-CONFIGS = {"P": P, "Q": Q, "R": R, "S": S}
-SEEDS = {"P": 11, "Q": 12, "R": 13, "S": 14}
+# T: nothing is a multiple of four: width 90, vocabulary 97, heads of 22 and 10, values of 18 and 14
+T = {"architecture": "Danonex", "vocab": 97, "width": 90, "norm": {"eps": 1e-5}, "residual_mult": 0.6,
+     "logit_scale": 1.5, "layers": [
+         layer(attention(3, 3, 22, 18, 0.5, softcap=9.0, rot_dims=10, base=50.0, scaling=YARN_A), ff=70),
+         layer(delta(3, 1, 10, 14, 3), ff=50),
+     ]}
+CONFIGS = {"P": P, "Q": Q, "R": R, "S": S, "T": T}
+SEEDS = {"P": 11, "Q": 12, "R": 13, "S": 14, "T": 15}
 
 STD = {"": 0.08, "embed": 0.5, "sink": 1.5, "A_log": 0.7, "dt_bias": 1.0, ".conv": 0.4, ".b": 0.3, ".a": 0.3}
 

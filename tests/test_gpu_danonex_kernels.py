@@ -275,3 +275,23 @@ def test_branch_norm_add_and_activations(dtype):
         got = x.to(DEV).clone()
         K.activation(got, kind)
         assert float((got.double().cpu() - fn(x.double())).abs().max()) <= (3e-6 if dtype == torch.float32 else 3e-2)
+
+
+@pytest.mark.parametrize("rows", [1, 8, 16, 40, 64])
+@pytest.mark.parametrize("kind", ["gelu", "gelu_tanh", "silu"])
+def test_the_few_row_product_with_an_activation_on_its_sums(rows, kind):
+    """act(a W^T) for up to 64 rows, the activation on the float32 sums: against the product in float64
+    and the plain activation, with one and with several ranges of k."""
+    K = _K()
+    gen = torch.Generator().manual_seed(rows)
+    a = torch.randn(rows, 256, generator=gen).bfloat16()
+    w = (torch.randn(328, 256, generator=gen) * 0.2).bfloat16()
+    z = a.double() @ w.double().T
+    fn = {"gelu": plain.gelu_erf, "silu": plain.silu,
+          "gelu_tanh": lambda t: 0.5 * t * (1 + torch.tanh(math.sqrt(2 / math.pi) * (t + 0.044715 * t ** 3)))}[kind]
+    want = fn(z)
+    for splits in (1, K.whole_sum_splits(328, 256, rows), 2):
+        out = torch.empty(rows, 328, dtype=torch.bfloat16, device=DEV)
+        K.gemm_skinny_act(out, a.to(DEV), w.to(DEV), kind, splits)
+        err = (out.double().cpu() - want).abs().max()
+        assert float(err) <= 2.0 ** -8 * float(want.abs().max()), (splits, float(err))
