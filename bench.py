@@ -66,14 +66,14 @@ def danonex_shape(shape: dict, layers: int) -> dict:
     one recurrent layer, every layer with a feed-forward."""
     heads, kv, hd = shape["num_attention_heads"], shape["num_key_value_heads"], shape["head_dim"]
     rot = {"base": float(shape["rope_theta"]), "dims": hd,
-           "scaling": {"factor": 4.0, "original": 8192, "fast": 32.0, "slow": 1.0}}
+           "scaling": {"factor": 8.0, "original": 4096, "fast": 16.0, "slow": 2.0}}
     attention = {"type": "attention", "mlp": {"kind": "dense", "ff": shape["intermediate_size"]},
-                 "mixer": {"heads": heads, "kv_heads": kv, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "softcap": 50.0,
+                 "mixer": {"heads": heads, "kv_heads": kv, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "softcap": 30.0,
                            "rot": rot}}
     recurrent = {"type": "delta", "mlp": {"kind": "dense", "ff": shape["intermediate_size"]},
                  "mixer": {"heads": heads, "kv_heads": max(1, heads // 2), "dim": hd, "vdim": hd, "conv": 4}}
     return {"architecture": "Danonex", "vocab": shape["vocab_size"], "width": shape["hidden_size"],
-            "norm": {"eps": shape["rms_norm_eps"]}, "residual_mult": 0.7, "logit_scale": 0.25,
+            "norm": {"eps": shape["rms_norm_eps"]}, "residual_mult": 0.5, "logit_scale": 0.5,
             "layers": [recurrent if i % 4 == 1 else attention for i in range(layers)]}
 
 

@@ -66,7 +66,7 @@ def tolerance(dtype, want):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,G,D,V,cap,bs", [(4, 2, 32, 32, 25.0, 16), (6, 2, 64, 64, 0.0, 16), (3, 1, 48, 80, 6.0, 16),
-                                            (2, 2, 96, 96, 30.0, 32), (5, 5, 20, 12, 0.0, 8)])
+                                            (2, 1, 160, 160, 30.0, 32), (5, 5, 20, 12, 0.0, 8)])
 def test_attention_with_cap_sinks_and_value_width(dtype, H, G, D, V, cap, bs):
     """A prompt of 700 tokens in one step, then single tokens: every query against the plain softmax.
     Query 699 and key 5 are scaled so that their score stands out (a far key among hundreds), queries
