@@ -45,6 +45,9 @@ def main(argv: Optional[List[str]] = None) -> int:
     p.add_argument("--stop-token-ids", default="", help='token ids that end a request, as "1,2"')
     p.add_argument("--max-num-seqs", type=int, default=None)
     p.add_argument("--max-num-batched-tokens", type=int, default=None)
+    p.add_argument("--num-state-slots", type=int, default=None,
+                   help="slots for per-request state of models with recurrent layers (default: --max-num-seqs, else "
+                        "one per prompt up to 256)")
     p.add_argument("--admission-margin-blocks", type=int, default=1)
     p.add_argument("--dump-logits", help="write every request's per-token logits to this .pt file")
     args = p.parse_args(argv)
@@ -63,7 +66,8 @@ def main(argv: Optional[List[str]] = None) -> int:
     options = dict(dtype=args.dtype, block_size=args.block_size, num_blocks=args.num_blocks, kv_bytes=args.kv_bytes,
                    fill_hbm=args.fill_hbm, max_num_seqs=args.max_num_seqs,
                    max_num_batched_tokens=args.max_num_batched_tokens,
-                   admission_margin_blocks=args.admission_margin_blocks, record_logits=bool(args.dump_logits))
+                   admission_margin_blocks=args.admission_margin_blocks, record_logits=bool(args.dump_logits),
+                   num_state_slots=args.num_state_slots, default_state_slots=min(len(prompts), 256))
     if args.random_config:
         with open(args.random_config) as handle:
             config = read_config_dict(json.load(handle))

@@ -37,11 +37,14 @@ class Engine:
                  max_num_batched_tokens: Optional[int] = None,
                  admission_margin_blocks: int = ADMISSION_MARGIN_BLOCKS, record_logits: bool = False,
                  device: str = "cuda:0", kv_bytes: Optional[int] = None, fill_hbm: Optional[float] = None,
-                 num_state_slots: Optional[int] = None) -> None:
+                 num_state_slots: Optional[int] = None, default_state_slots: Optional[int] = None) -> None:
         """`model`: a folder, or a built `Model`.  `dtype`: "bfloat16" or "float32"; None takes the
         folder's own (`torch_dtype` of its config.json), or the built model's.  The pool: `num_blocks`
         pages in every cache group (default 3,584), or `kv_bytes` for the whole cache, or `fill_hbm`,
-        the share of the device memory still free once the weights are in place."""
+        the share of the device memory still free once the weights are in place.  A model that keeps
+        per-request state (a recurrent mixer) has its slots allocated up front: `num_state_slots`, else
+        `max_num_seqs`, else `default_state_slots` (a caller that knows how many requests it will bring);
+        a model without such state ignores the last."""
         if isinstance(model, str):
             model = load_model(model, dtype, device)
         if dtype is None:
@@ -55,8 +58,11 @@ class Engine:
             raise ValueError(f"the engine was asked for {dtype} but the model it was given computes in {self.model.dtype}")
         self.num_blocks = self.config.pages(self.model.page_bytes(block_size), self._free_device_bytes)
         keeps_state = any(spec is not None for spec in self.model.cache_specs()[1])
-        self.cache = self.model.new_cache(block_size, self.num_blocks,
-                                          self.config.state_slots_for(self.num_blocks, keeps_state))
+        if keeps_state and num_state_slots is None and max_num_seqs is None and default_state_slots:
+            slots = int(default_state_slots)
+        else:
+            slots = self.config.state_slots_for(self.num_blocks, keeps_state)
+        self.cache = self.model.new_cache(block_size, self.num_blocks, slots)
         self.executor = ModelExecutor(self.model, self.cache)
         self.record_logits = record_logits
         self.scheduler = self._new_scheduler()
