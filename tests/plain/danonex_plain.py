@@ -114,12 +114,15 @@ def rotate_interleaved(x: torch.Tensor, positions: torch.Tensor, rot: dict, angl
 # --------------------------------------------------------------------------- mixers
 
 
-def attend(q, k, v, scale: float, cap, sinks, positions=None) -> torch.Tensor:
-    """q [T, H, D], k [T, G, D], v [T, G, V], sinks [H] or None -> [T, H, V]; query t sees keys 0..t."""
+def attend(q, k, v, scale: float, cap, sinks, positions=None, window=None) -> torch.Tensor:
+    """q [T, H, D], k [T, G, D], v [T, G, V], sinks [H] or None -> [T, H, V]; query t sees keys 0..t
+    (the design has no window; with one, for other designs that use these kernels, keys t-window+1..t)."""
     T, H = q.shape[0], q.shape[1]
     G, V = k.shape[1], v.shape[2]
     positions = torch.arange(T) if positions is None else positions
     causal = positions[None, :] <= positions[:, None]
+    if window:
+        causal = causal & (positions[:, None] - positions[None, :] < window)
     out = torch.zeros(T, H, V, dtype=q.dtype)
     for head in range(H):
         g = head // (H // G)

@@ -117,6 +117,42 @@ def test_attention_with_cap_sinks_and_value_width(dtype, H, G, D, V, cap, bs):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,G,D,V,bs", [(4, 2, 64, 64, 16), (3, 3, 24, 40, 16)])
+def test_capped_attention_with_sinks_inside_a_window(dtype, H, G, D, V, bs):
+    """The mechanisms together with a window (for designs that have one): the key just inside the window
+    of the last query and the one just outside it both stand out, and only the first may count."""
+    window, T = 100, 300
+    gen = torch.Generator().manual_seed(V)
+    q = torch.randn(T, H, D, generator=gen, dtype=torch.float64) * 0.5
+    k = torch.randn(T, G, D, generator=gen, dtype=torch.float64) * 0.5
+    v = torch.randn(T, G, V, generator=gen, dtype=torch.float64)
+    direction = torch.randn(D, generator=gen, dtype=torch.float64)
+    direction /= direction.norm()
+    q[T - 1] = 4.0 * direction
+    k[T - window] = 4.0 * direction        # the oldest key the last query sees
+    k[T - window - 1] = 6.0 * direction    # one further back: outside
+    sinks = torch.linspace(2.0, -2.0, H, dtype=torch.float64)
+    scale, cap = 2.0 / math.sqrt(D) * 3, 20.0
+    qr, kr, vr = (x.to(dtype).double() for x in (q, k, v))
+    want = plain.attend(qr, kr, vr, scale, cap, sinks, window=window).reshape(T, H * V)
+    table = scattered_table(-(-T // bs), 2, seed=1)
+    kc, vc = fill_cache(k, v, table, bs, dtype, spare=2)
+    tables, sink_dev = table.view(1, -1).to(DEV), sinks.float().to(DEV)
+    positions = torch.arange(T, dtype=torch.int32, device=DEV)
+    tok_seq = torch.zeros(T, dtype=torch.int32, device=DEV)
+    q_dev = q.to(dtype).reshape(T, H * D).to(DEV)
+    out = torch.empty(T, H * V, dtype=dtype, device=DEV)
+    attend(out, q_dev, kc, vc, positions, tok_seq, tables, [(0, 0, T, 0)], H, G, D, V, scale, window, cap, sink_dev)
+    assert float((out.double().cpu() - want).abs().max()) <= tolerance(dtype, want)
+    one = torch.empty(1, H * V, dtype=dtype, device=DEV)
+    attend(one, q_dev[T - 1:], kc, vc, positions[T - 1:], tok_seq[:1], tables, [(0, 0, 1, T - 1)], H, G, D, V, scale,
+           window, cap, sink_dev)
+    assert float((one.double().cpu()[0] - want[T - 1]).abs().max()) <= tolerance(dtype, want)
+    leaked = plain.attend(qr, kr, vr, scale, cap, sinks, window=window + 1).reshape(T, H * V)
+    assert float((leaked[T - 1] - want[T - 1]).abs().max()) > 5 * tolerance(dtype, want)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,G,D,V,rot,interleaved,norm", [(4, 2, 32, 16, 16, True, True), (3, 3, 48, 48, 48, True, True),
                                                             (2, 1, 64, 8, 32, False, True), (5, 1, 24, 40, 0, True, True),
                                                             (2, 2, 16, 16, 8, True, False)])
