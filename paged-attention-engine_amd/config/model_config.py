@@ -94,6 +94,15 @@ class MixerSpec(PartSpec):
     qk_norm_eps: float = 1e-6
     q_norm_name: str = "q_norm.weight"
     k_norm_name: str = "k_norm.weight"
+    # and some others' (a spec with any of these runs the mixer's convolution path):
+    # "head" as `qk_norm`: every query and key head divided by its own root mean square, no weight
+    mask: str = "window"                 # "chunk": `window` is a chunk length, position p sees keys from p - p % window on
+    conv_taps: Optional[int] = None      # a causal convolution over time on every channel of q, k and v, after the projection
+    conv_suffix: str = ".conv"           # its filters: <projection's name><suffix>, [channels, taps]
+    distance_slope_base: Optional[float] = None  # b: score -= 2^(-b (h + 1) / heads) * (query position - key position)
+    gate_name: Optional[str] = None      # a projection W_g of the mixer's input: heads *= sigmoid(W_g x) before W_o
+    bias_suffix: str = ".bias"
+    own_kv: bool = True                  # False: the layer has no key/value tensors at all; it reads another stop's cache
 
     @property
     def v_dim(self) -> int:
@@ -103,7 +112,43 @@ class MixerSpec(PartSpec):
     def plain(self) -> bool:
         """The reference's attention and nothing more: what the matrix-core kernels compute."""
         return (self.value_dim in (None, self.head_dim) and self.softcap is None and not self.sinks
-                and self.qk_norm is None)
+                and self.qk_norm is None and not self.convolved)
+
+    @property
+    def convolved(self) -> bool:
+        """Whether the spec takes the path with convolutions, per-head norms, distance bias, chunks or a gate."""
+        return (self.conv_taps is not None or self.qk_norm == "head" or self.mask != "window"
+                or self.distance_slope_base is not None or self.gate_name is not None or not self.own_kv)
+
+
+@dataclass(frozen=True)
+class LatentMixerSpec(PartSpec):
+    """Attention whose keys and values are products of one cached latent vector per token.
+
+    Per token the mixer's input is projected down to `kv_rank` + `rope_dim` features: the first
+    kv_rank, RMS-normed with a weight, are the latent c; the rest are one rotated key part shared by all
+    heads.  Head h's key is [W_uk_h c | rotated part], its value W_uv_h c; a query head has `nope_dim`
+    features that meet W_uk_h c and `rope_dim` rotated ones.  Only c and the rotated part are cached."""
+
+    hidden_size: int = 0
+    num_heads: int = 0
+    nope_dim: int = 0
+    rope_dim: int = 0
+    value_dim: int = 0
+    kv_rank: int = 0
+    scale: float = 1.0
+    window: Optional[int] = None
+    mask: str = "window"
+    position: Optional[PositionSpec] = None   # rotation of the rope_dim part (its rotary_dim <= rope_dim)
+    norm_eps: float = 1e-6
+    kind: str = "latent_attention"
+    q_name: str = "q"
+    down_name: str = "dkv"
+    down_norm_name: str = "dkv.norm"
+    up_k_name: str = "uk"
+    up_v_name: str = "uv"
+    o_name: str = "o"
+    weight_suffix: str = ""
 
 
 @dataclass(frozen=True)
@@ -164,6 +209,13 @@ class LayerSpec:
     feed_forward_norm_prefix: str = "post_attention_layernorm."
     arrangement: str = "prenorm"
     residual_scale: float = 1.0  # what a branch is multiplied by before it joins the stream ("branchnorm")
+    # arrangement "hyper": the stream is `streams` copies joined by hyper-connections whose tensors
+    # (in [S], out [S], mix [S, S] indexed [from, to]) lie under `connection_prefixes` (mixer, feed-forward;
+    # None: the plain sum x <- x + y), and a branch's output is first multiplied, feature by feature, by
+    # the tensors `layer_scale_names` (None: no such scale)
+    streams: int = 1
+    connection_prefixes: Optional[Tuple[str, str]] = None
+    layer_scale_names: Optional[Tuple[str, str]] = None
 
 
 @dataclass(frozen=True)
@@ -199,6 +251,7 @@ class ModelPlan:
     embedding_scale: float = 1.0            # the gathered rows are multiplied by this
     logit_scale: float = 1.0                # the logits are multiplied by this ...
     logit_softcap: Optional[float] = None   # ... and then, with a cap c, become c * tanh(logits / c)
+    streams: int = 1                        # copies the residual stream is kept in (blocks of arrangement "hyper")
     extra: Mapping[str, Any] = field(default_factory=dict)
 
     def __post_init__(self) -> None:
@@ -209,6 +262,11 @@ class ModelPlan:
                 raise ConfigError(
                     f"schedule entry {i} reads the cache of entry {entry.cache_from}, "
                     "which is not an earlier entry")
+        for i, layer in enumerate(self.layers):
+            if layer.streams != self.streams:
+                raise ConfigError(f"layer {i} keeps {layer.streams} copies of the stream, the model {self.streams}")
+            if layer.streams != 1 and layer.arrangement != "hyper":
+                raise ConfigError(f"layer {i}: only the arrangement 'hyper' keeps several copies of the stream")
         if self.logit_softcap is not None and not self.logit_softcap > 0:
             raise ConfigError(f"logit_softcap must be positive, got {self.logit_softcap}")
 

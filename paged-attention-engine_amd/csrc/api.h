@@ -29,6 +29,11 @@ int pae_rope_kv_write(int dtype, void* qkv, int64_t row_stride, int num_tokens, 
                       const void* bias, int b_is_f32, const float* cos_sin, const int* positions, const int* tok_seq, const int* block_tables,
                       int max_blocks, int bs, void* k_cache, void* v_cache, int write_kv, hipStream_t stream);
 int pae_swiglu(int dtype, void* out, const void* x, int num_tokens, int inter, int block, hipStream_t stream);
+int pae_gated_act(int dtype, void* out, const void* x, int num_tokens, int inter, int block, int kind,
+                  hipStream_t stream);  // act(gate) * up, act by code: 0 gelu (erf), 1 gelu (tanh), 2 silu
+int pae_gemm_plain_batched(int in_dtype, int out_dtype, void* C, int64_t ldc, int64_t batch_c, const void* A, int64_t lda,
+                           int64_t batch_a, const void* W, int64_t batch_w, const void* bias, int b_is_f32, int M, int N,
+                           int K, int batch, hipStream_t stream);
 int pae_gemm_plain(int in_dtype, int out_dtype, void* C, int64_t ldc, const void* A, int64_t lda, const void* W,
                    const void* bias, int b_is_f32, int M, int N, int K, hipStream_t stream);
 int pae_gemm_skinny(int epilogue, void* out, int64_t ldc, const void* A, int64_t lda, const void* W,
@@ -56,6 +61,31 @@ int pae_paged_attention_capped(int dtype, void* out, int64_t out_stride, const v
                                const void* k_cache, const void* v_cache, const int* positions, const int* tok_seq,
                                const int* block_tables, int max_blocks, int bs, int num_tokens, int nh, int nkv, int hd,
                                int vd, float scale, int window, float cap, const float* sinks, hipStream_t stream);
+// the same with a mask in chunks, a bias by distance, an output gate, and values shared with the keys
+int pae_paged_attention_masked(int dtype, void* out, int64_t out_stride, const void* q, int64_t q_stride,
+                               const void* k_cache, const void* v_cache, const int* positions, const int* tok_seq,
+                               const int* block_tables, int max_blocks, int bs, int num_tokens, int nh, int nkv, int hd,
+                               int vd, float scale, int window, float cap, const float* sinks, int chunked,
+                               const float* slopes, const void* gate, int64_t gate_stride, int shared_kv,
+                               hipStream_t stream);
+// a stream kept as several copies joined by hyper-connections: see hyper.hip
+int pae_hyper_norm(int dtype, float* streams, int num_streams, const void* y, int parts, int64_t part_stride,
+                   const void* ls, int ls_is_f32, const float* mix, const float* outw, const float* inw,
+                   const void* weight, int w_is_f32, float eps, const int* rows, void* out, int num_rows, int hidden,
+                   int write_back, hipStream_t stream);
+int pae_hyper_spread(float* streams, const float* src, int num_rows, int num_streams, int hidden, hipStream_t stream);
+int pae_hyper_collapse(float* out, const float* streams, int num_rows, int num_streams, int hidden, hipStream_t stream);
+// rows [q | k | v | ..]: short causal convolutions with per-request state, per-head RMS norm, cache write
+int pae_conv_norm_store(int dtype, const void* proj, int64_t row_stride, void* q_out, int64_t q_stride, int num_tokens,
+                        int num_seqs, const int* tok_seq, const int* positions, const int* seq_runs, const int* slots,
+                        const float* conv_w, float* conv_tail, int64_t tail_slot_stride, int taps, int nh, int nkv, int hd,
+                        int vd, int norm_heads, float eps, const int* block_tables, int max_blocks, int bs, void* k_cache,
+                        void* v_cache, hipStream_t stream);
+// rows [q heads of (nope + rd) | latent + rd]: latent norm, rotation, write of the latent pages: see latent.hip
+int pae_latent_prepare(int dtype, const void* proj, int64_t row_stride, void* q_full, int64_t qf_stride, int num_tokens,
+                       int nh, int nope, int rd, int rot, int interleaved, int rank, const void* norm_w, int w_is_f32,
+                       float eps, const float* cos_sin, const int* positions, const int* tok_seq, const int* block_tables,
+                       int max_blocks, int bs, void* latent, hipStream_t stream);
 // rows [q | k | v]: whole-projection RMS norm of q and of k (weights null: none), rotation, cache write
 int pae_qk_norm_rotate_store(int dtype, void* qkv, int64_t row_stride, int num_tokens, int nh, int nkv, int hd, int vd,
                              const void* q_w, const void* k_w, int w_is_f32, float eps, int rot, int interleaved,

@@ -514,6 +514,36 @@ __global__ void swiglu_vec8_kernel(bf16_t* __restrict__ out, const bf16_t* __res
   *reinterpret_cast<uint4*>(out + t * inter + j) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
 }
 
+// The gate with an activation by code (see act_of): out[t, j] = act(gate_j) * up_j, same layouts.
+template <typename T>
+__global__ void gated_act_kernel(T* __restrict__ out, const T* __restrict__ x, int inter, int block, int64_t total,
+                                 int kind) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const int64_t t = idx / inter;
+  const int j = (int)(idx % inter);
+  const int64_t gi = block ? (int64_t)(j / block) * 2 * block + j % block : j;
+  const int64_t ui = block ? gi + block : (int64_t)inter + j;
+  out[idx] = from_f32<T>(act_of(to_f32(x[t * 2 * inter + gi]), kind) * to_f32(x[t * 2 * inter + ui]));
+}
+
+extern "C" int pae_gated_act(int dtype, void* out, const void* x, int num_tokens, int inter, int block, int kind,
+                             hipStream_t stream) {
+  PAE_REQUIRE(num_tokens >= 0 && inter > 0, "gated_act: bad sizes T=%d I=%d", num_tokens, inter);
+  PAE_REQUIRE(block >= 0 && (block == 0 || inter % block == 0), "gated_act: blocks of %d do not divide %d", block, inter);
+  PAE_REQUIRE(kind >= 0 && kind <= 2, "gated_act: unknown activation code %d", kind);
+  const int64_t total = (int64_t)num_tokens * inter;
+  if (total == 0) return 0;
+  const unsigned blocks = (unsigned)((total + 255) / 256);
+  if (dtype == PAE_F32)
+    gated_act_kernel<float><<<blocks, 256, 0, stream>>>((float*)out, (const float*)x, inter, block, total, kind);
+  else if (dtype == PAE_BF16)
+    gated_act_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)x, inter, block, total, kind);
+  else
+    return pae_fail("gated_act: unknown dtype code %d", dtype);
+  return pae_check_launch("gated_act");
+}
+
 extern "C" int pae_swiglu(int dtype, void* out, const void* x, int num_tokens, int inter, int block,
                           hipStream_t stream) {
   PAE_REQUIRE(num_tokens >= 0 && inter > 0, "swiglu: bad sizes T=%d I=%d", num_tokens, inter);

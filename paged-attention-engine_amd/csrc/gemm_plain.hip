@@ -21,7 +21,12 @@ template <typename TA, typename TC>
 __global__ __launch_bounds__(256) void gemm_plain_kernel(TC* __restrict__ C, int64_t ldc,
                                                          const TA* __restrict__ A, int64_t lda,
                                                          const TA* __restrict__ W, const void* __restrict__ bias,
-                                                         int b_is_f32, int M, int N, int K) {
+                                                         int b_is_f32, int M, int N, int K,
+                                                         int64_t batch_c, int64_t batch_a, int64_t batch_w) {
+  // blockIdx.z: one of several products of equal sizes whose operands lie `batch_*` elements apart
+  C += blockIdx.z * batch_c;
+  A += blockIdx.z * batch_a;
+  W += blockIdx.z * batch_w;
   __shared__ float As[GP_BK][GP_BM + 4];
   __shared__ float Ws[GP_BK][GP_BN + 4];
   const int tid = threadIdx.x;
@@ -85,25 +90,34 @@ __global__ __launch_bounds__(256) void gemm_plain_kernel(TC* __restrict__ C, int
 }
 
 // in_dtype: operands; out_dtype: C.  Supported: f32->f32, bf16->bf16, bf16->f32.
-extern "C" int pae_gemm_plain(int in_dtype, int out_dtype, void* C, int64_t ldc, const void* A, int64_t lda,
-                              const void* W, const void* bias, int b_is_f32, int M, int N, int K,
-                              hipStream_t stream) {
+// `batch` products at once (one per head, say): product b reads A + b batch_a and W + b batch_w and
+// writes C + b batch_c, with the same leading dimensions; no bias then.
+extern "C" int pae_gemm_plain_batched(int in_dtype, int out_dtype, void* C, int64_t ldc, int64_t batch_c, const void* A,
+                                      int64_t lda, int64_t batch_a, const void* W, int64_t batch_w, const void* bias,
+                                      int b_is_f32, int M, int N, int K, int batch, hipStream_t stream) {
   PAE_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
+  PAE_REQUIRE(batch >= 1 && batch <= 65535 && (batch == 1 || !bias), "gemm: %d products at once (1..65535, no bias)", batch);
   PAE_REQUIRE(lda >= K && ldc >= N, "gemm: leading dimensions lda=%lld ldc=%lld too small for K=%d N=%d",
               (long long)lda, (long long)ldc, K, N);
   if (M == 0) return 0;
-  dim3 grid((N + GP_BN - 1) / GP_BN, (M + GP_BM - 1) / GP_BM);
+  dim3 grid((N + GP_BN - 1) / GP_BN, (M + GP_BM - 1) / GP_BM, batch);
   PAE_REQUIRE(grid.y <= 65535, "gemm: M=%d exceeds the grid", M);
   if (in_dtype == PAE_F32 && out_dtype == PAE_F32)
     gemm_plain_kernel<float, float><<<grid, 256, 0, stream>>>((float*)C, ldc, (const float*)A, lda,
-                                                              (const float*)W, bias, b_is_f32, M, N, K);
+                                                              (const float*)W, bias, b_is_f32, M, N, K, batch_c, batch_a, batch_w);
   else if (in_dtype == PAE_BF16 && out_dtype == PAE_BF16)
     gemm_plain_kernel<bf16_t, bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)C, ldc, (const bf16_t*)A, lda,
-                                                                (const bf16_t*)W, bias, b_is_f32, M, N, K);
+                                                                (const bf16_t*)W, bias, b_is_f32, M, N, K, batch_c, batch_a, batch_w);
   else if (in_dtype == PAE_BF16 && out_dtype == PAE_F32)
     gemm_plain_kernel<bf16_t, float><<<grid, 256, 0, stream>>>((float*)C, ldc, (const bf16_t*)A, lda,
-                                                               (const bf16_t*)W, bias, b_is_f32, M, N, K);
+                                                               (const bf16_t*)W, bias, b_is_f32, M, N, K, batch_c, batch_a, batch_w);
   else
     return pae_fail("gemm: unsupported dtype pair in=%d out=%d", in_dtype, out_dtype);
   return pae_check_launch("gemm_plain");
+}
+
+extern "C" int pae_gemm_plain(int in_dtype, int out_dtype, void* C, int64_t ldc, const void* A, int64_t lda,
+                              const void* W, const void* bias, int b_is_f32, int M, int N, int K,
+                              hipStream_t stream) {
+  return pae_gemm_plain_batched(in_dtype, out_dtype, C, ldc, 0, A, lda, 0, W, 0, bias, b_is_f32, M, N, K, 1, stream);
 }

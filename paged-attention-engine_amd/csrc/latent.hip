@@ -1,0 +1,87 @@
+// Latent attention: what is cached per token is one normed latent vector c (kv_rank wide) and one
+// rotated key part shared by all heads (rot_dim wide); keys and values of the heads are products of c.
+//
+// A projected row holds [q: nh heads of (nope + rd) | down: kv_rank + rd].  This kernel, one
+// workgroup per token:
+//   * divides the first kv_rank features of `down` by their root mean square (eps inside the root),
+//     multiplies by the norm's weight and writes them to the token's place in the latent pages,
+//     [block][offset][kv_rank + rd], features 0 .. kv_rank - 1;
+//   * rotates the first `rot` of the last rd features of `down` by the token's angles, pairs
+//     (2i, 2i + 1) if `interleaved` else (i, i + rot / 2), and writes all rd behind the latent;
+//   * rotates the last rd features of every query head likewise and writes them to
+//     q_full[t][head][kv_rank .. kv_rank + rd), where the attention kernel expects them behind the
+//     head's query folded into latent space (a product that the caller launches).
+// The attention over the pages then scores q_full against the cached row as a whole,
+//   score = q_folded . c + q_rotated . k_rotated,
+// and takes its values from the first kv_rank features of the same row.
+// Statistics, weights and the rotation are float32; a value is rounded to the storage type once.
+#include "common.h"
+#include "api.h"
+
+template <typename T>
+__global__ __launch_bounds__(256) void latent_prepare_kernel(
+    const T* __restrict__ proj, int64_t row_stride, T* __restrict__ q_full, int64_t qf_stride, int nh, int nope, int rd,
+    int rot, int interleaved, int rank, const void* __restrict__ norm_w, int w_is_f32, float eps,
+    const float* __restrict__ cos_sin, const int* __restrict__ positions, const int* __restrict__ tok_seq,
+    const int* __restrict__ block_tables, int max_blocks, int bs, T* __restrict__ latent) {
+  __shared__ float scratch[4];
+  const int t = blockIdx.x;
+  const T* row = proj + (int64_t)t * row_stride;
+  const T* down = row + (int64_t)nh * (nope + rd);
+  const int pos = positions[t];
+  const int64_t block = block_tables[(int64_t)tok_seq[t] * max_blocks + pos / bs];
+  T* cached = latent + (block * bs + pos % bs) * (int64_t)(rank + rd);
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < rank; i += 256) { const float x = to_f32(down[i]); ss = fmaf(x, x, ss); }
+  ss = block_sum<4>(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / (float)rank + eps);
+  for (int i = threadIdx.x; i < rank; i += 256)
+    cached[i] = from_f32<T>(to_f32(down[i]) * inv * load_param(norm_w, w_is_f32, i));
+  // rotated parts: "head" nh is the shared key part, heads 0 .. nh - 1 the queries'
+  const int half = rot / 2;
+  for (int idx = threadIdx.x; idx < (nh + 1) * half; idx += 256) {
+    const int h = idx / half, i = idx % half;
+    const int ia = interleaved ? 2 * i : i, ib = interleaved ? 2 * i + 1 : i + half;
+    const float c = cos_sin[((int64_t)t * half + i) * 2], s = cos_sin[((int64_t)t * half + i) * 2 + 1];
+    const T* src = h < nh ? row + (int64_t)h * (nope + rd) + nope : down + rank;
+    T* dst = h < nh ? q_full + (int64_t)t * qf_stride + (int64_t)h * (rank + rd) + rank : cached + rank;
+    const float a = to_f32(src[ia]), b = to_f32(src[ib]);
+    dst[ia] = from_f32<T>(a * c - b * s);
+    dst[ib] = from_f32<T>(b * c + a * s);
+  }
+  const int rest = rd - rot;  // features behind the rotated ones pass as they are
+  for (int idx = threadIdx.x; idx < (nh + 1) * rest; idx += 256) {
+    const int h = idx / rest, i = rot + idx % rest;
+    const T* src = h < nh ? row + (int64_t)h * (nope + rd) + nope : down + rank;
+    T* dst = h < nh ? q_full + (int64_t)t * qf_stride + (int64_t)h * (rank + rd) + rank : cached + rank;
+    dst[i] = src[i];
+  }
+}
+
+extern "C" int pae_latent_prepare(int dtype, const void* proj, int64_t row_stride, void* q_full, int64_t qf_stride,
+                                  int num_tokens, int nh, int nope, int rd, int rot, int interleaved, int rank,
+                                  const void* norm_w, int w_is_f32, float eps, const float* cos_sin, const int* positions,
+                                  const int* tok_seq, const int* block_tables, int max_blocks, int bs, void* latent,
+                                  hipStream_t stream) {
+  PAE_REQUIRE(nh > 0 && nope > 0 && rd >= 0 && rank > 0, "latent_prepare: bad sizes nh=%d nope=%d rd=%d rank=%d", nh, nope, rd,
+              rank);
+  PAE_REQUIRE(rot >= 0 && rot <= rd && rot % 2 == 0, "latent_prepare: %d rotated features of %d", rot, rd);
+  PAE_REQUIRE(rot == 0 || cos_sin, "latent_prepare: a rotation needs its table of cosines and sines");
+  PAE_REQUIRE(row_stride >= (int64_t)nh * (nope + rd) + rank + rd, "latent_prepare: row stride %lld too small",
+              (long long)row_stride);
+  PAE_REQUIRE(qf_stride >= (int64_t)nh * (rank + rd), "latent_prepare: query row stride %lld too small", (long long)qf_stride);
+  PAE_REQUIRE(bs > 0 && max_blocks > 0 && latent && block_tables && tok_seq && positions && norm_w && q_full,
+              "latent_prepare: missing operands");
+  if (num_tokens <= 0) return 0;
+  if (dtype == PAE_F32)
+    latent_prepare_kernel<float><<<num_tokens, 256, 0, stream>>>(
+        (const float*)proj, row_stride, (float*)q_full, qf_stride, nh, nope, rd, rot, interleaved, rank, norm_w, w_is_f32, eps,
+        cos_sin, positions, tok_seq, block_tables, max_blocks, bs, (float*)latent);
+  else if (dtype == PAE_BF16)
+    latent_prepare_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>(
+        (const bf16_t*)proj, row_stride, (bf16_t*)q_full, qf_stride, nh, nope, rd, rot, interleaved, rank, norm_w, w_is_f32,
+        eps, cos_sin, positions, tok_seq, block_tables, max_blocks, bs, (bf16_t*)latent);
+  else
+    return pae_fail("latent_prepare: unknown dtype code %d", dtype);
+  return pae_check_launch("latent_prepare");
+}

@@ -85,6 +85,7 @@ class Model:
         for block in self.blocks:
             block.bind(weights)
         self.final_norm.bind(plan.final_norm_prefix, weights)
+        self._sum_weights = torch.ones(plan.streams, dtype=torch.float32, device=self.device)
         if self.dtype == torch.bfloat16:
             K.skinny_tickets(self.device)  # made before any step is recorded as a graph
         if plan.head_name is None:
@@ -127,7 +128,9 @@ class Model:
             mixer = self.blocks[entry.layer].mixer
             borrowed = entry.cache_from is not None
             paged.append(None if borrowed else mixer.paged_spec())
-            states.append(None if borrowed else mixer.state_spec())
+            # a mixer that says so keeps state of its own at a stop that borrows its pages (the inputs of
+            # convolutions on its queries, say)
+            states.append(mixer.state_spec() if not borrowed or getattr(mixer, "state_when_borrowing", False) else None)
         return paged, states
 
     def page_bytes(self, block_size: int) -> int:
@@ -171,8 +174,14 @@ class Model:
         self.forward_pass_count += 1
         plan = self.plan
         T, H = ctx.num_tokens, plan.hidden_size
+        copies = plan.streams
         residual = torch.empty((T, H), dtype=torch.float32, device=self.device)
         stream = ResidualStream(residual)
+        if copies > 1:
+            # the stream is kept in several copies, all equal to the embedding's output at the start
+            stream = ResidualStream(torch.empty((T, copies * H), dtype=torch.float32, device=self.device))
+            stream.copies = copies
+        stream.sum_weights = self._sum_weights
         # the norm that reads the stream first at every stop (and the final norm after the last)
         first_norms = [getattr(self.blocks[entry.layer], "mixer_norm", None) for entry in plan.schedule] + [self.final_norm]
         entry_fold = getattr(self.blocks[plan.schedule[0].layer], "entry_fold", None) if plan.schedule and T else None
@@ -186,6 +195,8 @@ class Model:
             stream.owed, stream.owed_to = OwedRows(rows, stats, eps), norm
         else:
             K.embedding(residual, self.embedding, token_ids, plan.embedding_scale)
+            if copies > 1:
+                K.hyper_spread(stream.residual, residual, copies)
         program = ctx.program if fold is not None and self.decode_fusable(ctx) else None
         if program is not None:
             # every block's kernels become phases of one resident kernel, which runs when all are recorded

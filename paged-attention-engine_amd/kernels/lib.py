@@ -72,6 +72,14 @@ def _declare(lib) -> None:
         "pae_paged_attention_generic": [I, P, L, P, L, P, P, P, P, P, I, I, I, I, I, I, F, I, P],
         "pae_paged_attention_capped": [I, P, L, P, L, P, P, P, P, P, I, I, I, I, I, I, I, F, I, F, P, P],
         "pae_qk_norm_rotate_store": [I, P, L, I, I, I, I, I, P, P, I, F, I, I, P, F, P, P, P, I, I, P, P, I, P],
+        "pae_paged_attention_masked": [I, P, L, P, L, P, P, P, P, P, I, I, I, I, I, I, I, F, I, F, P, I, P, P, L, I, P],
+        "pae_hyper_norm": [I, P, I, P, I, L, P, I, P, P, P, P, I, F, P, P, I, I, I, P],
+        "pae_hyper_spread": [P, P, I, I, I, P],
+        "pae_hyper_collapse": [P, P, I, I, I, P],
+        "pae_conv_norm_store": [I, P, L, P, L, I, I, P, P, P, P, P, P, L, I, I, I, I, I, I, F, P, I, I, P, P, P],
+        "pae_latent_prepare": [I, P, L, P, L, I, I, I, I, I, I, I, P, I, F, P, P, P, P, I, I, P, P],
+        "pae_gated_act": [I, P, P, I, I, I, I, P],
+        "pae_gemm_plain_batched": [I, I, P, L, L, P, L, L, P, L, P, I, I, I, I, I, P],
         "pae_rows_from_residual": [I, P, P, L, P],
         "pae_norm_scale_add": [I, P, P, I, L, P, I, F, F, P, I, I, P],
         "pae_activation": [I, P, L, I, P],
@@ -306,6 +314,17 @@ def swiglu(out: torch.Tensor, x: torch.Tensor, block: int = 0) -> None:
     T, I = out.shape
     assert x.shape == (T, 2 * I) and x.dtype == out.dtype and x.is_contiguous() and out.is_contiguous()
     _check(library().pae_swiglu(code_of(x.dtype), out.data_ptr(), x.data_ptr(), T, I, block, _stream()))
+
+
+def gated_act(out: torch.Tensor, x: torch.Tensor, kind: str, block: int = 0) -> None:
+    """`swiglu` with the gate's activation by name (see ACTIVATIONS): out = act(gate) * up."""
+    _not_while_recording("gated_act")
+    _gpu(out, x)
+    T, I = out.shape
+    assert x.shape == (T, 2 * I) and x.dtype == out.dtype and x.is_contiguous() and out.is_contiguous()
+    assert kind in ACTIVATIONS
+    _check(library().pae_gated_act(code_of(x.dtype), out.data_ptr(), x.data_ptr(), T, I, block, ACTIVATIONS[kind],
+                                   _stream()))
 
 
 # ---------------------------------------------------------------------------------- decode programs
@@ -869,6 +888,26 @@ def gemm_plain(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Option
                                     a.data_ptr(), a.stride(0), w.data_ptr(), bp, bf, M, N, K, _stream()))
 
 
+def gemm_plain_heads(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor) -> None:
+    """One product per head: out[:, h, :] = a[:, h, :] @ w[h]^T, float32 accumulation in k order.
+    `a` [M, B, K] and `out` [M, B, N] are views whose last dimension is contiguous (heads of wider
+    rows, say); `w` [B, N, K] is contiguous."""
+    _not_while_recording("gemm_plain_heads")
+    _gpu(out, a, w)
+    M, B, K = a.shape
+    N = w.shape[1]
+    assert w.shape == (B, N, K) and w.is_contiguous() and w.dtype == a.dtype
+    assert out.shape == (M, B, N) and a.stride(2) == 1 and out.stride(2) == 1
+    _check(library().pae_gemm_plain_batched(code_of(a.dtype), code_of(out.dtype), out.data_ptr(), out.stride(0),
+                                            out.stride(1), a.data_ptr(), a.stride(0), a.stride(1), w.data_ptr(),
+                                            w.stride(0), None, 0, M, N, K, B, _stream()))
+
+
+def heads_product(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor) -> None:
+    """out[:, h, :] = a[:, h, :] @ w[h]^T for every head h (shapes as for `gemm_plain_heads`)."""
+    gemm_plain_heads(out, a, w)
+
+
 def paged_attention_generic(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                             positions: torch.Tensor, tok_seq: torch.Tensor, block_tables: torch.Tensor,
                             nh: int, nkv: int, hd: int, scale: float, window: int) -> None:
@@ -921,6 +960,176 @@ def paged_attention_capped(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Te
         v_cache.data_ptr(), positions.data_ptr(), tok_seq.data_ptr(), block_tables.data_ptr(),
         block_tables.shape[1], bs, T, nh, nkv, hd, vd, float(scale), int(window), float(softcap), _ptr(sinks),
         _stream()))
+
+
+def paged_attention_masked(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: Optional[torch.Tensor],
+                           positions: torch.Tensor, tok_seq: torch.Tensor, block_tables: torch.Tensor,
+                           nh: int, nkv: int, hd: int, vd: int, scale: float, window: int = 0, chunked: bool = False,
+                           slopes: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
+                           softcap: float = 0.0, sinks: Optional[torch.Tensor] = None) -> None:
+    """`paged_attention_capped` with, each optional: the `window` read as a chunk length (`chunked`:
+    position p sees keys from p - p % window on), a bias by distance (score -= slopes[h] * (p - key),
+    float32 [nh]), and an output gate (out *= sigmoid(gate), `gate` a [T, >= nh * vd] view of rows).
+    `v_cache` None: the values are the first `vd` features of the key rows, which are then one row
+    per token, `k_cache` [block][bs][hd] (nkv must be 1)."""
+    _not_while_recording("paged_attention_masked")
+    _gpu(out, q, k_cache, v_cache, positions, tok_seq, block_tables, sinks, slopes, gate)
+    T = q.shape[0]
+    assert q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= nh * hd and q.dtype == k_cache.dtype == out.dtype
+    assert out.shape[0] == T and out.stride(1) == 1 and out.shape[1] >= nh * vd
+    if v_cache is None:
+        assert nkv == 1 and k_cache.dim() == 3 and k_cache.shape[2] == hd and k_cache.is_contiguous() and vd <= hd
+        bs = k_cache.shape[1]
+    else:
+        bs = k_cache.shape[2]
+        _check_pools_wide(k_cache, v_cache, nkv, bs, hd, vd)
+    assert positions.dtype == torch.int32 and positions.numel() == T
+    assert tok_seq.dtype == torch.int32 and tok_seq.numel() == T
+    assert block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous()
+    for t in (sinks, slopes):
+        if t is not None:
+            assert t.dtype == torch.float32 and t.numel() == nh and t.is_contiguous()
+    gate_stride = 0
+    if gate is not None:
+        assert gate.dim() == 2 and gate.shape[0] == T and gate.stride(1) == 1 and gate.shape[1] >= nh * vd
+        assert gate.dtype == q.dtype
+        gate_stride = gate.stride(0)
+    _check(library().pae_paged_attention_masked(
+        code_of(q.dtype), out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0), k_cache.data_ptr(),
+        _ptr(v_cache), positions.data_ptr(), tok_seq.data_ptr(), block_tables.data_ptr(),
+        block_tables.shape[1], bs, T, nh, nkv, hd, vd, float(scale), int(window), float(softcap), _ptr(sinks),
+        1 if chunked else 0, _ptr(slopes), _ptr(gate), gate_stride, 1 if v_cache is None else 0, _stream()))
+
+
+def conv_norm_store(proj: torch.Tensor, q_out: torch.Tensor, tok_seq: torch.Tensor, positions: torch.Tensor,
+                    seq_runs: torch.Tensor, slots: torch.Tensor, conv_w: torch.Tensor, conv_tail: Optional[torch.Tensor],
+                    taps: int, nh: int, nkv: int, hd: int, vd: int, norm_heads: bool, eps: float,
+                    block_tables: Optional[torch.Tensor], block_size: int, k_cache: Optional[torch.Tensor],
+                    v_cache: Optional[torch.Tensor]) -> None:
+    """Rows `proj` [T, >= C], C = nh hd + nkv (hd + vd), hold per token [q | k | v | anything else]:
+    every one of the C channels passes a causal convolution of `taps` taps over the sequence's own
+    tokens (`conv_w` float32 [C, taps]; inputs before the step from `conv_tail` float32
+    [slots, taps - 1, C], which is moved on), then, with `norm_heads`, q and k heads are divided by
+    their root mean square over hd.  Queries to `q_out` [T, nh * hd], keys and values to their cache
+    slots (nkv = 0: queries only, no pools).  `seq_runs` int32 [S, 4] = (first row, rows, tokens
+    before, 0) per sequence."""
+    _not_while_recording("conv_norm_store")
+    _gpu(proj, q_out, tok_seq, positions, seq_runs, slots, conv_w, conv_tail, block_tables, k_cache, v_cache)
+    T, S = proj.shape[0], seq_runs.shape[0]
+    C = nh * hd + nkv * (hd + vd)
+    assert proj.dim() == 2 and proj.stride(1) == 1 and proj.shape[1] >= C
+    assert q_out.shape == (T, nh * hd) and q_out.stride(1) == 1 and q_out.dtype == proj.dtype
+    for t, n in ((tok_seq, T), (positions, T), (slots, S)):
+        assert t.dtype == torch.int32 and t.numel() >= n and t.is_contiguous()
+    assert seq_runs.dtype == torch.int32 and seq_runs.shape == (S, 4) and seq_runs.is_contiguous()
+    assert seq_runs.data_ptr() % 16 == 0
+    assert conv_w.dtype == torch.float32 and conv_w.shape == (C, taps) and conv_w.is_contiguous()
+    tail_stride = 0
+    if taps > 1:
+        assert conv_tail is not None and conv_tail.dtype == torch.float32
+        assert tuple(conv_tail.shape[1:]) == (taps - 1, C) and conv_tail[0].is_contiguous()
+        tail_stride = conv_tail.stride(0)
+    max_blocks = 0
+    if nkv:
+        assert k_cache.dtype == proj.dtype == v_cache.dtype
+        assert block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous()
+        assert block_tables.shape[0] >= S
+        _check_pools_wide(k_cache, v_cache, nkv, block_size, hd, vd)
+        max_blocks = block_tables.shape[1]
+    _check(library().pae_conv_norm_store(
+        code_of(proj.dtype), proj.data_ptr(), proj.stride(0), q_out.data_ptr(), q_out.stride(0), T, S,
+        tok_seq.data_ptr(), positions.data_ptr(), seq_runs.data_ptr(), slots.data_ptr(), conv_w.data_ptr(),
+        _ptr(conv_tail) if taps > 1 else None, tail_stride, taps, nh, nkv, hd, vd, 1 if norm_heads else 0, float(eps),
+        _ptr(block_tables) if nkv else None, max_blocks, block_size, _ptr(k_cache) if nkv else None,
+        _ptr(v_cache) if nkv else None, _stream()))
+
+
+def latent_prepare(proj: torch.Tensor, q_full: torch.Tensor, nh: int, nope: int, rd: int, rot: int, interleaved: bool,
+                   rank: int, norm_w: torch.Tensor, eps: float, cos_sin: Optional[torch.Tensor], positions: torch.Tensor,
+                   tok_seq: torch.Tensor, block_tables: torch.Tensor, latent: torch.Tensor) -> None:
+    """Rows `proj` [T, nh (nope + rd) + rank + rd] = [query heads | down projection]: the first `rank`
+    features of the down projection are RMS-normed with `norm_w` and, with the last rd (their first
+    `rot` rotated by `cos_sin`), written to the token's row of `latent` [block][bs][rank + rd]; the
+    query heads' last rd features are rotated likewise into q_full[t, h, rank:] (`q_full`
+    [T, nh * (rank + rd)], whose first `rank` features per head the caller fills)."""
+    _not_while_recording("latent_prepare")
+    _gpu(proj, q_full, norm_w, cos_sin, positions, tok_seq, block_tables, latent)
+    T = proj.shape[0]
+    assert proj.dim() == 2 and proj.stride(1) == 1 and proj.shape[1] >= nh * (nope + rd) + rank + rd
+    assert q_full.shape == (T, nh * (rank + rd)) and q_full.stride(1) == 1 and q_full.dtype == proj.dtype
+    assert latent.dim() == 3 and latent.shape[2] == rank + rd and latent.is_contiguous() and latent.dtype == proj.dtype
+    assert positions.dtype == torch.int32 and positions.numel() == T
+    assert tok_seq.dtype == torch.int32 and tok_seq.numel() == T
+    assert block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous()
+    assert norm_w.numel() == rank and norm_w.is_contiguous()
+    _check_cos_sin(cos_sin, rot, T)
+    wp, wf = _param(norm_w)
+    _check(library().pae_latent_prepare(
+        code_of(proj.dtype), proj.data_ptr(), proj.stride(0), q_full.data_ptr(), q_full.stride(0), T, nh, nope, rd, rot,
+        1 if interleaved else 0, rank, wp, wf, float(eps), _ptr(cos_sin) if rot else None, positions.data_ptr(),
+        tok_seq.data_ptr(), block_tables.data_ptr(), block_tables.shape[1], latent.shape[1], latent.data_ptr(), _stream()))
+
+
+def hyper_norm(streams: torch.Tensor, num_streams: int, y: Optional[torch.Tensor], layer_scale: Optional[torch.Tensor],
+               mix: Optional[torch.Tensor], out_weights: Optional[torch.Tensor], in_weights: torch.Tensor,
+               weight: torch.Tensor, eps: float, out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> None:
+    """A stream kept as `num_streams` float32 copies per token (`streams` [T, S * H]).  With `y`, the
+    pending branch output ([T, H] in out's dtype, or float32 partial sums [P, T, H]), all copies move
+    on at once: x_t <- sum_s mix[s, t] x_s + out_weights[t] * (layer_scale * y).  Then
+    out = rmsnorm(sum_s in_weights[s] x_s) * weight.  `mix` [S, S], `out_weights` and `in_weights` [S]
+    are float32.  With `rows` (int32) only those rows are produced and nothing is written back."""
+    _not_while_recording("hyper_norm")
+    _gpu(streams, y, layer_scale, mix, out_weights, in_weights, weight, out, rows)
+    S = num_streams
+    T = streams.shape[0]
+    H = out.shape[-1]
+    n = out.shape[0]
+    assert streams.dtype == torch.float32 and streams.is_contiguous() and tuple(streams.shape) == (T, S * H)
+    assert out.is_contiguous() and weight.numel() == H
+    assert in_weights.dtype == torch.float32 and in_weights.numel() == S and in_weights.is_contiguous()
+    parts, part_stride = 0, 0
+    if y is not None:
+        assert y.is_contiguous()
+        if y.dim() == 3:
+            assert y.dtype == torch.float32 and tuple(y.shape[1:]) == (T, H)
+            parts, part_stride = y.shape[0], T * H
+        else:
+            assert y.dtype == out.dtype and tuple(y.shape) == (T, H)
+        assert mix.dtype == torch.float32 and tuple(mix.shape) == (S, S) and mix.is_contiguous()
+        assert out_weights.dtype == torch.float32 and out_weights.numel() == S and out_weights.is_contiguous()
+        if layer_scale is not None:
+            assert layer_scale.numel() == H and layer_scale.is_contiguous()
+    if rows is None:
+        assert n == T
+    else:
+        assert rows.dtype == torch.int32 and rows.numel() == n
+    lp, lf = _param(layer_scale if y is not None else None)
+    wp, wf = _param(weight)
+    _check(library().pae_hyper_norm(code_of(out.dtype), streams.data_ptr(), S, _ptr(y), parts, part_stride, lp, lf,
+                                    _ptr(mix) if y is not None else None, _ptr(out_weights) if y is not None else None,
+                                    in_weights.data_ptr(), wp, wf, float(eps), _ptr(rows), out.data_ptr(), n, H,
+                                    0 if rows is not None else 1, _stream()))
+
+
+def hyper_spread(streams: torch.Tensor, src: torch.Tensor, num_streams: int) -> None:
+    """streams[t] = `num_streams` copies of src[t] (float32 [T, H] -> [T, S * H])."""
+    _not_while_recording("hyper_spread")
+    _gpu(streams, src)
+    T, H = src.shape
+    assert src.dtype == torch.float32 == streams.dtype and src.is_contiguous() and streams.is_contiguous()
+    assert tuple(streams.shape) == (T, num_streams * H)
+    _check(library().pae_hyper_spread(streams.data_ptr(), src.data_ptr(), T, num_streams, H, _stream()))
+
+
+def hyper_collapse(streams: torch.Tensor, num_streams: int) -> torch.Tensor:
+    """The sum of a token's copies: float32 [T, S * H] -> [T, H]."""
+    _not_while_recording("hyper_collapse")
+    _gpu(streams)
+    T, H = streams.shape[0], streams.shape[1] // num_streams
+    assert streams.dtype == torch.float32 and streams.is_contiguous() and streams.shape[1] == num_streams * H
+    out = torch.empty((T, H), dtype=torch.float32, device=streams.device)
+    _check(library().pae_hyper_collapse(out.data_ptr(), streams.data_ptr(), T, num_streams, H, _stream()))
+    return out
 
 
 def qk_norm_rotate_store(qkv: torch.Tensor, nh: int, nkv: int, hd: int, vd: int, q_weight: Optional[torch.Tensor],

@@ -24,18 +24,30 @@ softcap * tanh(score / softcap), and a learned sink per query head that joins th
 denominator as exp(sink) without a key or a value (`sinks`).  A spec with any of them takes the
 path `_forward_wide`: the projection, then one kernel that norms, rotates and stores, then the
 attention kernel that knows caps, sinks and value widths.
+
+And for designs that have them (`MixerSpec.convolved`, the path `_forward_convolved`): a short causal
+convolution over time on every channel of q, k and v right after the projection, whose last
+taps - 1 inputs are per-request state next to the pages; every query and key head divided by its own
+root mean square (`qk_norm = "head"`, no weight); a bias by distance instead of a rotation,
+score -= 2^(-b (h + 1) / H) * (i - j); a mask in chunks counted from position 0 of the sequence
+(`mask = "chunk"`); a gate sigmoid(W_g x) on the concatenated heads before W_o, whose projection is
+part of the one product and which the attention kernel applies as it writes; and layers without
+key/value tensors that read an earlier layer's pages (`own_kv = False`).  Pages of such a layer are
+never handed back early: a reader with another mask may still want them.
 """
 
 from __future__ import annotations
 
 import torch
 
-from ..cache.manager import attention_pages
+from ..cache.manager import StateSpec, attention_pages
 from ..kernels import lib as K
 from .base import POSITION_ENCODINGS, OwedRows, Part, ScaleShape, StepShape, build_part, plain_rows, register_mixer
+from .delta import sequence_runs
 from .linear import Linear, rows_a_graph_may_hold
 
 WORK_LISTS = ("paged attention work lists", K.PREFILL_TILE)
+CONV_LISTS = ("paged attention work lists and sequence runs", K.PREFILL_TILE)
 
 
 def attention_work_lists(shape: StepShape):
@@ -85,9 +97,21 @@ class PagedAttention(Part):
             raise ValueError(f"head_dim {spec.head_dim}: the attention kernels take multiples of 16 up to 256")
         if not spec.plain and not (0 < spec.head_dim <= 1024 and 0 < spec.v_dim <= 256):
             raise ValueError(f"head_dim {spec.head_dim} / value_dim {spec.v_dim}: the attention kernel takes up to 1024 / 256")
-        if spec.qk_norm not in (None, "projection"):
-            raise ValueError(f"qk_norm '{spec.qk_norm}' is not known (known: projection)")
-        if not spec.plain and (spec.qkv_bias or spec.out_bias):
+        if spec.qk_norm not in (None, "projection", "head"):
+            raise ValueError(f"qk_norm '{spec.qk_norm}' is not known (known: projection, head)")
+        if spec.mask not in ("window", "chunk"):
+            raise ValueError(f"mask '{spec.mask}' is not known (known: window, chunk)")
+        if spec.convolved:
+            if spec.position is not None or spec.qk_norm == "projection" or spec.sinks or spec.softcap:
+                raise ValueError("an attention with convolutions, per-head norms, chunks, distance bias or a gate "
+                                 "takes no rotation, projection norm, sinks or cap")
+            if spec.conv_taps is not None and not 1 <= spec.conv_taps <= 64:
+                raise ValueError(f"conv_taps {spec.conv_taps} is outside 1..64")
+            if spec.mask == "chunk" and not spec.window:
+                raise ValueError("a mask in chunks needs the chunk length (window)")
+        elif not spec.own_kv:
+            raise ValueError("only the convolution path knows layers without key/value tensors")
+        if not spec.plain and not spec.convolved and (spec.qkv_bias or spec.out_bias):
             raise ValueError("an attention with value widths, caps, sinks or query/key norms takes no biases")
         self.position = (build_part(POSITION_ENCODINGS, "position encoding", spec.position, dtype, device)
                          if spec.position is not None else
@@ -115,8 +139,22 @@ class PagedAttention(Part):
                 and K.program_takes_product(rows, s.num_heads * s.head_dim, K.residual_splits(
                     s.hidden_size, s.num_heads * s.head_dim, rows)))
 
+    state_when_borrowing = True  # the convolution on the queries has inputs to remember at every stop
+
     def paged_spec(self):
-        return attention_pages(self.spec.num_kv_heads, self.spec.head_dim, self.spec.window, self.spec.value_dim)
+        s = self.spec
+        return attention_pages(s.num_kv_heads, s.head_dim, None if s.convolved else s.window, s.value_dim)
+
+    @property
+    def conv_channels(self) -> int:
+        s = self.spec
+        return s.num_heads * s.head_dim + (s.num_kv_heads * (s.head_dim + s.v_dim) if s.own_kv else 0)
+
+    def state_spec(self):
+        taps = self.spec.conv_taps
+        if not taps or taps < 2:
+            return None
+        return StateSpec((taps - 1, self.conv_channels), torch.float32, "conv_tail")
 
     def _matrix_cores(self, block_size: int) -> bool:
         s = self.spec
@@ -124,13 +162,38 @@ class PagedAttention(Part):
                 and K.mfma_attention_supported(self.dtype, s.num_heads, s.num_kv_heads, s.head_dim, block_size))
 
     def step_lists_key(self, block_size: int):
+        if self.spec.convolved:
+            return CONV_LISTS
         return WORK_LISTS if self._matrix_cores(block_size) else None
 
     def step_lists(self, shape: StepShape):
+        if self.spec.convolved:
+            return {**attention_work_lists(shape), **sequence_runs(shape)}
         return attention_work_lists(shape)
+
+    def _projections(self):
+        """(name, rows) of the projections that pass the convolution, in the order of the product's columns."""
+        s = self.spec
+        out = [(s.q_name, s.num_heads * s.head_dim)]
+        if s.own_kv:
+            out += [(s.k_name, s.num_kv_heads * s.head_dim), (s.v_name, s.num_kv_heads * s.v_dim)]
+        return out
 
     def tensors(self, prefix):
         s = self.spec
+        if s.convolved:
+            out = {prefix + s.o_name + s.weight_suffix: (s.hidden_size, s.num_heads * s.v_dim)}
+            for name, rows in self._projections():
+                out[prefix + name + s.weight_suffix] = (rows, s.hidden_size)
+                if s.qkv_bias:
+                    out[prefix + name + s.bias_suffix] = (rows,)
+                if s.conv_taps is not None:
+                    out[prefix + name + s.conv_suffix] = (rows, s.conv_taps)
+            if s.gate_name is not None:
+                out[prefix + s.gate_name + s.weight_suffix] = (s.num_heads * s.v_dim, s.hidden_size)
+            if s.out_bias:
+                out[prefix + s.o_name + s.bias_suffix] = (s.hidden_size,)
+            return out
         out = {prefix + s.q_name + s.weight_suffix: (s.num_heads * s.head_dim, s.hidden_size),
                prefix + s.k_name + s.weight_suffix: (s.num_kv_heads * s.head_dim, s.hidden_size),
                prefix + s.v_name + s.weight_suffix: (s.num_kv_heads * s.v_dim, s.hidden_size),
@@ -148,8 +211,32 @@ class PagedAttention(Part):
             out[prefix + s.o_name + ".bias"] = (s.hidden_size,)
         return out
 
+    def _bind_convolved(self, prefix, weights):
+        s = self.spec
+        f32 = dict(device=self.device, dtype=torch.float32)
+        named = self._projections()
+        parts = [weights[prefix + name + s.weight_suffix] for name, _ in named]
+        bias = [weights[prefix + name + s.bias_suffix] for name, _ in named] if s.qkv_bias else None
+        if s.gate_name is not None:  # the gate reads the same input: its rows ride in the same product, without a bias
+            parts.append(weights[prefix + s.gate_name + s.weight_suffix])
+            if bias is not None:
+                bias.append(torch.zeros(s.num_heads * s.v_dim, dtype=bias[0].dtype, device=bias[0].device))
+        self.qkv = Linear(self.matrix(torch.cat(parts, dim=0)), None if bias is None else self.vector(torch.cat(bias, dim=0)))
+        if s.conv_taps is not None:
+            self.conv = torch.cat([weights[prefix + name + s.conv_suffix] for name, _ in named], dim=0).to(**f32).contiguous()
+        else:
+            self.conv = torch.ones((self.conv_channels, 1), **f32)
+        ob = weights[prefix + s.o_name + s.bias_suffix] if s.out_bias else None
+        self.out = Linear(self.matrix(weights[prefix + s.o_name + s.weight_suffix]), None if ob is None else self.vector(ob))
+        self.slopes = None
+        if s.distance_slope_base is not None:
+            h = torch.arange(1, s.num_heads + 1, dtype=torch.float64)
+            self.slopes = torch.pow(2.0, -float(s.distance_slope_base) * h / s.num_heads).to(**f32).contiguous()
+
     def bind(self, prefix, weights):
         s = self.spec
+        if s.convolved:
+            return self._bind_convolved(prefix, weights)
         names = (s.q_name, s.k_name, s.v_name)
         w = torch.cat([weights[prefix + n + s.weight_suffix] for n in names], dim=0)
         b = (torch.cat([weights[prefix + n + ".bias"] for n in names], dim=0) if s.qkv_bias else None)
@@ -229,9 +316,39 @@ class PagedAttention(Part):
                      s.num_kv_heads, s.head_dim, s.v_dim, s.scale, s.window or 0, s.softcap or 0.0, self.sinks)
         return self.out.branch(attn, ctx.sink)
 
+    def _forward_convolved(self, ctx, x):
+        """The path of a spec that is `convolved`: one product [q | k | v | gate], one kernel that
+        convolves, norms the heads and stores, and the attention kernel that knows chunks, the distance
+        bias and the gate."""
+        s = self.spec
+        if s.own_kv != ctx.writes_cache:
+            raise ValueError("a layer with key/value tensors writes its own pages, one without reads another stop's")
+        pages = ctx.cache.pages_of(ctx.cache_entry)
+        table = ctx.block_tables[ctx.cache.group_of(ctx.cache_entry)]
+        proj = self.qkv(x)
+        nkv = s.num_kv_heads if s.own_kv else 0
+        taps = s.conv_taps or 1
+        lists = ctx.memo[CONV_LISTS]
+        q = torch.empty((proj.shape[0], s.num_heads * s.head_dim), dtype=proj.dtype, device=proj.device)
+        K.conv_norm_store(proj, q, ctx.tok_seq, ctx.positions, lists["runs"], ctx.slots, self.conv,
+                          ctx.cache.state_of(ctx.entry) if taps > 1 else None, taps, s.num_heads, nkv, s.head_dim, s.v_dim,
+                          s.qk_norm == "head", s.qk_norm_eps, table if nkv else None, ctx.cache.block_size,
+                          pages["k"] if nkv else None, pages["v"] if nkv else None)
+        gate = None
+        if s.gate_name is not None:
+            first = self.conv_channels
+            gate = proj[:, first:first + s.num_heads * s.v_dim]
+        attn = torch.empty((proj.shape[0], s.num_heads * s.v_dim), dtype=proj.dtype, device=proj.device)
+        K.paged_attention_masked(attn, q, pages["k"], pages["v"], ctx.positions, ctx.tok_seq, table, s.num_heads,
+                                 s.num_kv_heads, s.head_dim, s.v_dim, s.scale, s.window or 0, s.mask == "chunk",
+                                 self.slopes, gate)
+        return self.out.branch(attn, ctx.sink)
+
     def forward(self, ctx, x):
         """`x`: normalised activations, or `OwedRows` (the projection then pays their scale)."""
         s = self.spec
+        if s.convolved:
+            return self._forward_convolved(ctx, plain_rows(x))
         if not s.plain:
             return self._forward_wide(ctx, plain_rows(x))
         pages = ctx.cache.pages_of(ctx.cache_entry)  # as declared in `paged_spec`

@@ -88,6 +88,20 @@ class ResidualStream:
         # is such a block and will want them (set by the model)
         self.rows: Optional[torch.Tensor] = None
         self.rows_wanted_next = False
+        # for blocks that keep the stream in several copies (`residual` is then [T, copies * H]): how
+        # `pending` joins them (a `StreamJoin`), and the weights of a read that is their plain sum
+        self.copies = 1
+        self.join: Optional["StreamJoin"] = None
+        self.sum_weights: Optional[torch.Tensor] = None
+
+
+class StreamJoin:
+    """How a pending branch output joins a stream that is kept in several copies: every copy t becomes
+    sum_s mix[s, t] x_s + out[t] * (scale * y), `scale` one factor per feature (None: none).  `mix`
+    [S, S] and `out` [S] are float32 on the device."""
+
+    def __init__(self, mix: torch.Tensor, out: torch.Tensor, scale: Optional[torch.Tensor]) -> None:
+        self.mix, self.out, self.scale = mix, out, scale
 
 
 class BranchSink:

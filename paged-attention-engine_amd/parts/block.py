@@ -7,8 +7,8 @@ left pending on the stream and added by the next norm, in float32.
 
 from __future__ import annotations
 
-from .base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, BranchSink, Part, ResidualStream, build_part, plain_rows,
-                   register_block)
+from .base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, BranchSink, Part, ResidualStream, ScaleShape, StreamJoin,
+                   build_part, plain_rows, register_block)
 
 
 @register_block("prenorm")
@@ -154,6 +154,105 @@ class BranchNormBlock:
         if has_ff:
             y = self.feed_forward.forward(ctx, self._rows(stream))
             self._join(stream, self.feed_forward_out_norm, y, follows)
+
+
+@register_block("hyper")
+class HyperBlock:
+    """Pre-norm branches on a stream that is kept in S copies x_1 .. x_S (hyper-connections), each
+    branch's output scaled feature by feature before it joins (layer scale).  For sublayer q
+    (mixer, then feed-forward) with its tensors in [S], out [S] and mix [S, S] (indexed [from, to]):
+
+        u = sum_s in[s] x_s;   y = scale_q * sublayer(norm_q(u));   x_t <- sum_s mix[s, t] x_s + out[t] y
+
+    for all t at once from the old copies.  Without connection tensors (`connection_prefixes` None)
+    the copies are one and the join is x <- x + y; without `layer_scale_names` there is no scale; a
+    layer whose spec names no feed-forward has the first half only.  The copies are float32.  A
+    branch's output is left pending on the stream with the way it joins (`StreamJoin`), and the norm
+    that reads the stream next does join, read and norm in one kernel."""
+
+    def __init__(self, layer_spec, dtype, device):
+        self.spec = layer_spec
+        self.dtype, self.device = dtype, device
+        self.copies = int(layer_spec.streams)
+        if layer_spec.connection_prefixes is None and self.copies != 1:
+            raise ValueError(f"{self.copies} copies of the stream need connection tensors to join them")
+        self.mixer_norm = build_part(NORMS, "norm", layer_spec.mixer_norm, dtype, device)
+        self.mixer = build_part(MIXERS, "mixer", layer_spec.mixer, dtype, device)
+        self.feed_forward = self.feed_forward_norm = None
+        if layer_spec.feed_forward is not None:
+            self.feed_forward_norm = build_part(NORMS, "norm", layer_spec.feed_forward_norm, dtype, device)
+            self.feed_forward = build_part(FEED_FORWARDS, "feed-forward", layer_spec.feed_forward, dtype, device)
+        for norm in (self.mixer_norm, self.feed_forward_norm):
+            if norm is not None and not hasattr(norm, "forward_copies"):
+                raise ValueError(f"the norm '{norm.spec.kind}' cannot read a stream of several copies (no forward_copies)")
+        self.reads = [None, None]   # float32 [S]: how each sublayer reads the copies
+        self.joins = [None, None]   # StreamJoin: how each sublayer's output joins them
+
+    def _named(self):
+        s = self.spec
+        out = [(self.mixer_norm, s.prefix + s.mixer_norm_prefix), (self.mixer, s.prefix + s.mixer_prefix)]
+        if self.feed_forward is not None:
+            out += [(self.feed_forward_norm, s.prefix + s.feed_forward_norm_prefix),
+                    (self.feed_forward, s.prefix + s.feed_forward_prefix)]
+        return out
+
+    def _sublayers(self):
+        return (0, 1) if self.feed_forward is not None else (0,)
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(part.graph_safe for part, _ in self._named())
+
+    @property
+    def graph_max_rows(self):
+        limits = [part.graph_max_rows for part, _ in self._named() if part.graph_max_rows is not None]
+        return min(limits) if limits else None
+
+    def parts(self):
+        return [part for part, _ in self._named()]
+
+    def tensors(self):
+        s, S = self.spec, self.copies
+        out = {}
+        for part, prefix in self._named():
+            out.update(part.tensors(prefix))
+        for q in self._sublayers():
+            if s.connection_prefixes is not None:
+                at = s.prefix + s.connection_prefixes[q]
+                out[at + "in"] = (S,)
+                out[at + "out"] = (S,)
+                out[at + "mix"] = (S, S)
+            if s.layer_scale_names is not None:
+                out[s.prefix + s.layer_scale_names[q]] = ScaleShape((s.mixer_norm.size,))
+        return out
+
+    def bind(self, weights):
+        import torch
+        s, S = self.spec, self.copies
+        for part, prefix in self._named():
+            part.bind(prefix, weights)
+        f32 = dict(device=self.device, dtype=torch.float32)
+        for q in self._sublayers():
+            if s.connection_prefixes is not None:
+                at = s.prefix + s.connection_prefixes[q]
+                read = weights[at + "in"].to(**f32).contiguous()
+                mix, out = weights[at + "mix"].to(**f32).contiguous(), weights[at + "out"].to(**f32).contiguous()
+            else:
+                read, mix, out = (torch.ones(shape, **f32) for shape in ((1,), (1, 1), (1,)))
+            scale = None
+            if s.layer_scale_names is not None:  # the scale enters the residual sum, which is float32
+                scale = weights[s.prefix + s.layer_scale_names[q]].to(**f32).contiguous()
+            self.reads[q], self.joins[q] = read, StreamJoin(mix, out, scale)
+
+    def forward(self, ctx, stream: ResidualStream) -> None:
+        if stream.owed is not None or stream.copies != self.copies:
+            raise ValueError("a block on a stream of several copies follows one that left the stream in another form")
+        ctx.sink = None
+        x = self.mixer_norm.forward_copies(stream, self.reads[0])
+        stream.pending, stream.join = self.mixer.forward(ctx, x), self.joins[0]
+        if self.feed_forward is not None:
+            x = self.feed_forward_norm.forward_copies(stream, self.reads[1])
+            stream.pending, stream.join = self.feed_forward.forward(ctx, x), self.joins[1]
 
 
 def build_block(layer_spec, dtype, device):

@@ -1,0 +1,116 @@
+"""Latent attention: keys and values of all heads are products of one cached vector per token.
+
+Per token, with h the mixer's input:  q = W_q h, head by head [nope_dim unrotated | rope_dim rotated];
+W_down h has kv_rank + rope_dim rows: the first kv_rank, RMS-normed with a weight, are the latent c,
+the last rope_dim are one key part shared by all heads.  Head j's key is [W_uk_j c | shared part], its
+value W_uv_j c; query and shared key part are rotated by position; the score is
+
+    (q_nope . W_uk_j c + q_rot . k_rot) * scale
+
+over the keys the mask lets through (a sliding window, chunks, or every earlier key), an ordinary
+softmax, and W_o on the concatenated heads.
+
+Only c and the rotated part are cached, one row of kv_rank + rope_dim per token whatever the number
+of heads (`paged_spec`: one tensor "latent" [PAGE][kv_rank + rope_dim]).  The heads' keys and values
+are never formed: since q_nope . (W_uk_j c) = (W_uk_j^T q_nope) . c, the query is folded into latent
+space once per token ([W_uk_j^T q_nope | q_rot], kv_rank + rope_dim wide), the attention kernel scores
+it against the cached row as it is and sums the rows' first kv_rank features as values, and the
+head's output is W_uv_j times that sum.  The query projection and the down projection are one
+product; the two per-head products are one launch each.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from ..cache.manager import PAGE, PagedSpec, PagedTensor
+from ..kernels import lib as K
+from .base import POSITION_ENCODINGS, Part, ScaleShape, build_part, plain_rows, register_mixer
+from .linear import Linear, rows_a_graph_may_hold
+
+
+def latent_pages(kv_rank: int, rope_dim: int, window=None) -> PagedSpec:
+    """One row per token: the latent vector, then the rotated key part."""
+    return PagedSpec((PagedTensor("latent", (PAGE, kv_rank + rope_dim)),), window)
+
+
+@register_mixer("latent_attention")
+class LatentAttention(Part):
+    def __init__(self, spec, dtype, device):
+        super().__init__(spec, dtype, device)
+        if min(spec.num_heads, spec.nope_dim, spec.value_dim, spec.kv_rank) <= 0 or spec.rope_dim < 0:
+            raise ValueError("latent attention: heads, nope_dim, value_dim and kv_rank must be positive")
+        if spec.kv_rank + spec.rope_dim > 1024 or spec.kv_rank > 512:
+            raise ValueError(f"latent attention: kv_rank {spec.kv_rank} + rope_dim {spec.rope_dim}: the kernels take "
+                             "rows up to 1024 with a latent up to 512")
+        if spec.mask not in ("window", "chunk"):
+            raise ValueError(f"mask '{spec.mask}' is not known (known: window, chunk)")
+        if spec.mask == "chunk" and not spec.window:
+            raise ValueError("a mask in chunks needs the chunk length (window)")
+        rotated = getattr(spec.position, "rotary_dim", 0) if spec.position is not None else 0
+        if rotated > spec.rope_dim:
+            raise ValueError(f"{rotated} rotated features of a rotated part of {spec.rope_dim}")
+        self.position = (build_part(POSITION_ENCODINGS, "position encoding", spec.position, dtype, device)
+                         if spec.position is not None else POSITION_ENCODINGS["none"](None, dtype, device))
+        if not hasattr(self.position, "rotary_table") or float(getattr(self.position, "magnitude", 1.0)) != 1.0:
+            raise ValueError("latent attention rotates by a plain table of cosines and sines")
+
+    @property
+    def graph_safe(self) -> bool:
+        return self.position.graph_safe
+
+    @property
+    def graph_max_rows(self):
+        s = self.spec
+        return rows_a_graph_may_hold(self.dtype, s.hidden_size, s.num_heads * s.value_dim)
+
+    @property
+    def row_width(self) -> int:
+        return self.spec.kv_rank + self.spec.rope_dim
+
+    def paged_spec(self):
+        s = self.spec
+        return latent_pages(s.kv_rank, s.rope_dim, s.window if s.mask == "window" else None)
+
+    def tensors(self, prefix):
+        s = self.spec
+        sfx = s.weight_suffix
+        return {prefix + s.q_name + sfx: (s.num_heads * (s.nope_dim + s.rope_dim), s.hidden_size),
+                prefix + s.down_name + sfx: (self.row_width, s.hidden_size),
+                prefix + s.down_norm_name: ScaleShape((s.kv_rank,)),
+                prefix + s.up_k_name + sfx: (s.num_heads * s.nope_dim, s.kv_rank),
+                prefix + s.up_v_name + sfx: (s.num_heads * s.value_dim, s.kv_rank),
+                prefix + s.o_name + sfx: (s.hidden_size, s.num_heads * s.value_dim)}
+
+    def bind(self, prefix, weights):
+        s = self.spec
+        sfx = s.weight_suffix
+        self.proj = Linear(self.matrix(torch.cat([weights[prefix + s.q_name + sfx], weights[prefix + s.down_name + sfx]],
+                                                 dim=0)))
+        self.down_norm = self.vector(weights[prefix + s.down_norm_name])
+        up_k = weights[prefix + s.up_k_name + sfx].view(s.num_heads, s.nope_dim, s.kv_rank)
+        # the fold q_nope -> W_uk^T q_nope is a product with W_uk^T as its [out, in] matrix, head by head
+        self.up_k_t = self.matrix(up_k.transpose(1, 2))
+        self.up_v = self.matrix(weights[prefix + s.up_v_name + sfx].view(s.num_heads, s.value_dim, s.kv_rank))
+        self.out = Linear(self.matrix(weights[prefix + s.o_name + sfx]))
+
+    def forward(self, ctx, x):
+        s = self.spec
+        if not ctx.writes_cache:
+            raise ValueError("a latent attention layer keeps pages of its own")
+        x = plain_rows(x)
+        T, H, C, R, D, V = x.shape[0], s.num_heads, s.kv_rank, s.rope_dim, s.nope_dim, s.value_dim
+        latent = ctx.cache.pages_of(ctx.cache_entry)["latent"]
+        table = ctx.block_tables[ctx.cache.group_of(ctx.cache_entry)]
+        proj = self.proj(x)
+        rot, cos_sin = self.position.rotary_table(ctx)
+        q_full = torch.empty((T, H * (C + R)), dtype=proj.dtype, device=proj.device)
+        K.latent_prepare(proj, q_full, H, D, R, rot, bool(getattr(self.position, "interleaved", False)), C,
+                         self.down_norm, s.norm_eps, cos_sin, ctx.positions, ctx.tok_seq, table, latent)
+        K.heads_product(q_full.view(T, H, C + R)[:, :, :C], proj[:, :H * (D + R)].view(T, H, D + R)[:, :, :D], self.up_k_t)
+        summed = torch.empty((T, H * C), dtype=proj.dtype, device=proj.device)
+        K.paged_attention_masked(summed, q_full, latent, None, ctx.positions, ctx.tok_seq, table, H, 1, C + R, C, s.scale,
+                                 s.window or 0, s.mask == "chunk")
+        heads = torch.empty((T, H * V), dtype=proj.dtype, device=proj.device)
+        K.heads_product(heads.view(T, H, V), summed.view(T, H, C), self.up_v)
+        return self.out.branch(heads, ctx.sink)

@@ -1,5 +1,6 @@
-"""Feed-forwards.  "swiglu", the dense gated one: down(silu(gate(x)) * up(x)), no biases
-(engine/model.py:317-320 of the reference).  gate and up are one product over
+"""Feed-forwards.  "swiglu", the dense gated one: down(act(gate(x)) * up(x)), no biases, act = silu
+(engine/model.py:317-320 of the reference) or another of `kernels.lib.ACTIVATIONS` by the spec's
+`activation`.  gate and up are one product over
 concatenated weights; the gate is applied in float32 and rounded once.  "dense", the plain
 one: down(act(up(x))), act one of `kernels.lib.ACTIVATIONS`, applied in float32."""
 
@@ -18,8 +19,9 @@ class SwiGLU(Part):
     takes_owed_rows = True
     def __init__(self, spec, dtype, device):
         super().__init__(spec, dtype, device)
-        if spec.activation != "silu":
-            raise ValueError(f"activation '{spec.activation}' is not supported by the gated feed-forward")
+        if spec.activation not in K.ACTIVATIONS:
+            raise ValueError(f"activation '{spec.activation}' is not one of {', '.join(K.ACTIVATIONS)}")
+        self.silu = spec.activation == "silu"  # the activation the few-row product's gated epilogue knows
 
     @property
     def graph_max_rows(self):
@@ -49,7 +51,7 @@ class SwiGLU(Part):
 
     def decode_fusable(self, rows: int, block_size: int) -> bool:
         s = self.spec
-        return (self.dtype == torch.bfloat16 and bool(self.block) and 0 < rows <= K.program_max_rows()
+        return (self.silu and self.dtype == torch.bfloat16 and bool(self.block) and 0 < rows <= K.program_max_rows()
                 and s.hidden_size % 8 == 0 and s.intermediate_size % 8 == 0
                 and K.program_takes_product(rows, s.hidden_size,
                                             K.whole_sum_splits(2 * s.intermediate_size, s.hidden_size, rows))
@@ -60,12 +62,14 @@ class SwiGLU(Part):
         """`x`: normalised activations, or `OwedRows` (the gated product then pays their scale)."""
         act = torch.empty((x.shape[0], self.spec.intermediate_size), dtype=x.dtype, device=x.device)
         rows = x.rows if isinstance(x, OwedRows) else x
-        if self.block and x.shape[0] and K.skinny_supported(rows, self.gate_up.weight):
+        if self.silu and self.block and x.shape[0] and K.skinny_supported(rows, self.gate_up.weight):
             splits = K.whole_sum_splits(2 * self.spec.intermediate_size, self.spec.hidden_size, x.shape[0])
             K.gemm_skinny(act, rows, self.gate_up.weight, None, K.EPI_SWIGLU, splits,
                           row_scale=x.row_scale if isinstance(x, OwedRows) else None)
-        else:
+        elif self.silu:
             K.swiglu(act, self.gate_up(plain_rows(x)), self.block)
+        else:
+            K.gated_act(act, self.gate_up(plain_rows(x)), self.spec.activation, self.block)
         return self.down.branch(act, getattr(ctx, "sink", None))
 
 

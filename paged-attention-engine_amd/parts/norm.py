@@ -43,6 +43,8 @@ class RMSNorm(Part):
         rows.  With `rows` (int32 indices) only those rows are produced and the
         stream is left untouched.  When the branch before has added itself into the residual
         and prepared this norm's rows, they are returned as they are (`OwedRows`): no kernel runs."""
+        if stream.copies > 1 or stream.join is not None:
+            return self.forward_copies(stream, stream.sum_weights, rows)
         if stream.owed is not None:
             owed, mine = stream.owed, stream.owed_to is self
             if rows is None:
@@ -55,6 +57,23 @@ class RMSNorm(Part):
         K.add_rmsnorm(stream.residual, stream.pending, self.weight, self.spec.eps, out, rows)
         if rows is None:
             stream.pending = None
+        return out
+
+    def forward_copies(self, stream: ResidualStream, read_weights: torch.Tensor,
+                       rows: Optional[torch.Tensor] = None):
+        """The norm on a stream kept in several copies: the pending branch joins them as `stream.join`
+        says, then the row sum_s read_weights[s] x_s is normed.  Sum and norm are float32 and the
+        result is rounded once.  With `rows` only those rows are produced and the stream stays as it is."""
+        n = stream.residual.shape[0] if rows is None else rows.numel()
+        out = torch.empty((n, self.spec.size), dtype=self.dtype, device=stream.residual.device)
+        join = stream.join if stream.pending is not None else None
+        if stream.pending is not None and join is None:
+            raise ValueError("a branch is pending on a stream of several copies without the way it joins them")
+        K.hyper_norm(stream.residual, stream.copies, stream.pending if join else None, join.scale if join else None,
+                     join.mix if join else None, join.out if join else None, read_weights, self.weight, self.spec.eps,
+                     out, rows)
+        if rows is None:
+            stream.pending = stream.join = None
         return out
 
     def add_scaled(self, residual: torch.Tensor, y: torch.Tensor, scale: float,
