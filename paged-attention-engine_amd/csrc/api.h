@@ -123,6 +123,18 @@ int pae_attn_prefill_capped_bf16(void* out, int64_t out_stride, const void* q, i
                                  const void* v_cache, const int* tiles, int num_tiles, const int* positions,
                                  const int* block_tables, int max_blocks, int bs, int nh, int nkv, int hd, float scale,
                                  int window, float cap, const float* sinks, hipStream_t stream);
+// the two with the window read as a chunk length (`chunked`), a bias by distance (`slopes` float32 [nh] or null:
+// score -= slopes[h] (position - key)) and a gate on the output (`gate` bfloat16 rows [token][nh * hd] or null)
+int pae_attn_decode_biased_bf16(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* k_cache,
+                                const void* v_cache, const int* dec_work, int num_dec, const int* block_tables,
+                                int max_blocks, int bs, int nh, int nkv, int hd, float scale, int window, int chunked,
+                                const float* slopes, const void* gate, int64_t gate_stride, void* part_acc, void* part_ml,
+                                hipStream_t stream);
+int pae_attn_prefill_biased_bf16(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* k_cache,
+                                 const void* v_cache, const int* tiles, int num_tiles, const int* positions,
+                                 const int* block_tables, int max_blocks, int bs, int nh, int nkv, int hd, float scale,
+                                 int window, int chunked, const float* slopes, const void* gate, int64_t gate_stride,
+                                 hipStream_t stream);
 // A decode step's layers as one resident kernel (see decode_program.hip).
 // A caller builds a list of phases in host memory with the put functions (each returns the bytes of
 // LDS a quad of four wavefronts needs for the phase, or a negative code), copies it to the device and

@@ -34,11 +34,13 @@ __device__ __forceinline__ float tanh_fast(float x) {
 // value feature 0 of the tile's first key (feature stride `vstride` elements).
 // q[ct][j]: B operand of column tile ct for hd slice j.  pos/start: per lane's column.
 // CAPPED: scores are capped, s <- cap tanh(s / cap): `cap_log2` = cap log2(e), `scale_over_cap` = scale / cap.
-template <int HD, int CT, bool CAPPED = false>
+// BIASED: a bias by distance, score -= slope (position - key): `slope_log2` = the column's slope times log2(e).
+template <int HD, int CT, bool CAPPED = false, bool BIASED = false>
 __device__ __forceinline__ void attn_tile(AttnState<HD, CT>& st, const bf16x8 (&kf)[HD / 32],
                                           const s16x4 (&vf)[HD / 16], const bf16x8 (&q)[CT][HD / 32],
                                           int key0, const int (&pos)[CT], const int (&start)[CT],
-                                          float scale_log2, float cap_log2 = 0.f, float scale_over_cap = 0.f) {
+                                          float scale_log2, float cap_log2 = 0.f, float scale_over_cap = 0.f,
+                                          float slope_log2 = 0.f) {
   const int g4 = threadIdx.x % PAE_WAVE / 16;
 #pragma unroll
   for (int ct = 0; ct < CT; ++ct) {
@@ -49,7 +51,8 @@ __device__ __forceinline__ void attn_tile(AttnState<HD, CT>& st, const bf16x8 (&
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int key = key0 + 4 * g4 + i;
-      const float scaled = CAPPED ? cap_log2 * tanh_fast(s[i] * scale_over_cap) : s[i] * scale_log2;
+      float scaled = CAPPED ? cap_log2 * tanh_fast(s[i] * scale_over_cap) : s[i] * scale_log2;
+      if (BIASED) scaled -= slope_log2 * (float)(pos[ct] - key);
       s[i] = (key <= pos[ct] && key >= start[ct]) ? scaled : -INFINITY;
       mx = fmaxf(mx, s[i]);
     }

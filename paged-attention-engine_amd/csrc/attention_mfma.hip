@@ -25,6 +25,10 @@
 // Masking is the reference's rule (engine/attention.py:474-487: key j visible iff
 // j <= position of the query) plus an optional window.  A column's result depends
 // only on its own position: fully masked pages add exact zeros.
+//
+// For designs that have them (the BIASED instantiations): the window read as a chunk length
+// (`chunked`: position p sees the keys from p - p % window on), a bias by distance,
+// score -= slopes[head] (p - key), and a gate on the output, out *= sigmoid(gate[token][head][feature]).
 #include "common.h"
 #include "api.h"
 #include "attention_device.h"
@@ -39,13 +43,19 @@
 // for every workgroup and cost more than the second launch.)
 //   part_acc[((token * nkv + kvh) * max_splits + split) * g + head in group][HD]
 //   part_ml [ ... same index ... ][2] = (maximum in log2 units, sum)
-template <int HD, int TPW, bool CAPPED>
+__device__ __forceinline__ int first_visible(int pos, int window, int chunked) {
+  if (window <= 0) return 0;
+  if (chunked) return pos - pos % window;
+  return pos - window + 1 > 0 ? pos - window + 1 : 0;
+}
+
+template <int HD, int TPW, bool CAPPED, bool BIASED>
 __global__ __launch_bounds__(256) void attn_decode_kernel(
     float* __restrict__ part_acc, float* __restrict__ part_ml, int max_splits,
     const bf16_t* __restrict__ q, int64_t q_stride,
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache, const int4* __restrict__ dec_work,
     const int* __restrict__ block_tables, int max_blocks, int bs, int nh, int nkv, float scale_log2, int window,
-    float cap_log2, float scale_over_cap) {
+    float cap_log2, float scale_over_cap, int chunked, const float* __restrict__ slopes) {
   constexpr int SPLIT = 64 * TPW;
   const int split = blockIdx.x, kvh = blockIdx.y;
   // one load brings the token's row, its position and its table row: a chain of three dependent
@@ -63,7 +73,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   }
   const int tok = work.x;
   const int pos[1] = {work.y};
-  const int start[1] = {(window > 0 && pos[0] - window + 1 > 0) ? pos[0] - window + 1 : 0};
+  const int start[1] = {BIASED ? first_visible(pos[0], window, chunked)
+                               : ((window > 0 && pos[0] - window + 1 > 0) ? pos[0] - window + 1 : 0)};
   const int s_first = start[0] / SPLIT, s_last = pos[0] / SPLIT;
   if (split < s_first || split > s_last) return;
   const int lo = max(split * SPLIT, start[0] / 16 * 16);
@@ -89,6 +100,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   st.l[0] = 0.f;
 #pragma unroll
   for (int t = 0; t < HD / 16; ++t) st.acc[0][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  const float slope_log2 = (BIASED && slopes) ? slopes[kvh * g + (col < g ? col : 0)] * LOG2E : 0.f;
 
   const int page_elems = bs * HD;
   const int tile_lo = lo / 16, tile_hi = (hi + 15) / 16;
@@ -107,7 +119,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     const int tile = tile_lo + wave + 4 * j;
     keys_to_mfma_order<HD>(kf[j]);  // in every lane of the wavefront, used or not
     if (tile < tile_hi)
-      attn_tile<HD, 1, CAPPED>(st, kf[j], vf[j], qf, tile * 16, pos, start, scale_log2, cap_log2, scale_over_cap);
+      attn_tile<HD, 1, CAPPED, BIASED>(st, kf[j], vf[j], qf, tile * 16, pos, start, scale_log2, cap_log2, scale_over_cap,
+                                       slope_log2);
   }
 
   // wavefronts 1..3 hand their state to wavefront 0 through LDS; every lane of a wavefront
@@ -162,7 +175,8 @@ template <int HD, int TPW>
 __global__ void attn_decode_merge_kernel(bf16_t* __restrict__ out, int64_t out_stride,
                                          const float* __restrict__ part_acc, const float* __restrict__ part_ml,
                                          int max_splits, const int4* __restrict__ dec_work, int nh, int nkv,
-                                         int window, const float* __restrict__ sinks) {
+                                         int window, const float* __restrict__ sinks, int chunked,
+                                         const bf16_t* __restrict__ gate, int64_t gate_stride) {
   // blockDim = (items rounded up to wavefronts, G): the splits are dealt out to G groups of threads,
   // whose loads are all in flight together; group 0 then adds the groups' sums in group order.
   extern __shared__ float s_merge[];  // [G - 1][items][6]: four sums, maximum, sum of weights
@@ -170,7 +184,7 @@ __global__ void attn_decode_merge_kernel(bf16_t* __restrict__ out, int64_t out_s
   const int kvh = blockIdx.x;
   const int4 work = dec_work[blockIdx.y];
   const int tok = work.x, pos = work.y;
-  const int start = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int start = first_visible(pos, window, chunked);
   const int s_first = start / SPLIT, nsplits = pos / SPLIT - s_first + 1;
   const int g = nh / nkv, items = g * (HD / 4);
   const int item = threadIdx.x, group = threadIdx.y, groups = blockDim.y;  // item: (head in group, four features)
@@ -216,8 +230,14 @@ __global__ void attn_decode_merge_kernel(bf16_t* __restrict__ out, int64_t out_s
   }
   const float inv = 1.0f / l;
   s16x4 w;
+  if (gate) {
+    const bf16_t* gt = gate + (int64_t)tok * gate_stride + (int64_t)(kvh * g + c) * HD + d;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) w[i] = bf16_bits(a[i] * inv);
+    for (int i = 0; i < 4; ++i) w[i] = bf16_bits(a[i] * inv / (1.0f + expf(-__bfloat162float(gt[i]))));
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) w[i] = bf16_bits(a[i] * inv);
+  }
   *reinterpret_cast<s16x4*>(out + (int64_t)tok * out_stride + (int64_t)(kvh * g + c) * HD + d) = w;
 }
 
@@ -254,12 +274,13 @@ __device__ __forceinline__ bf16x8 quad_to_mfma_order(bf16x8 x, int fetch_from) {
 // tiles[t] = (table row of the sequence, first flat token, number of tokens <= 64); blockIdx.z picks
 // the part of 16 CT tokens of the run that this workgroup takes.
 // BS: the page size if it is 16 (the value rows' offsets are then constants), or 0 for any other.
-template <int HD, int CT, int BS, bool CAPPED>
+template <int HD, int CT, int BS, bool CAPPED, bool BIASED>
 __global__ __launch_bounds__(256, 1) void attn_prefill_split_kernel(
     bf16_t* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ q, int64_t q_stride,
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache, const int* __restrict__ tiles,
     const int* __restrict__ positions, const int* __restrict__ block_tables, int max_blocks, int bs, int nh,
-    int nkv, float scale_log2, int window, float cap_over_scale, float scale_over_cap, const float* __restrict__ sinks) {
+    int nkv, float scale_log2, int window, float cap_over_scale, float scale_over_cap, const float* __restrict__ sinks,
+    int chunked, const float* __restrict__ slopes, float inv_scale, const bf16_t* __restrict__ gate, int64_t gate_stride) {
   constexpr int UNIT = 32, TOK = 16 * CT;
   if (BS) bs = BS;
   __shared__ float s_acc[3][HD / 16][4][PAE_WAVE];
@@ -272,6 +293,7 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_split_kernel(
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / PAE_WAVE), lane = threadIdx.x % PAE_WAVE;
   const int col = lane % 16, g4 = lane / 16;
   const int head = blockIdx.x, kvh = head / (nh / nkv);
+  const float slope_over_scale = (BIASED && slopes) ? slopes[head] * inv_scale : 0.f;
   const int seq_row = tiles[blockIdx.y * 3];
   const int tok0 = tiles[blockIdx.y * 3 + 1] + blockIdx.z * TOK;
   const int ntok = min(TOK, tiles[blockIdx.y * 3 + 2] - (int)blockIdx.z * TOK);
@@ -285,7 +307,8 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_split_kernel(
     const int c = ct * 16 + col;
     const bool live = c < ntok;
     pos[ct] = live ? pos0 + c : -1;  // a dead column sees no key
-    start[ct] = (live && window > 0 && pos[ct] - window + 1 > 0) ? pos[ct] - window + 1 : 0;
+    if (BIASED) start[ct] = live ? first_visible(pos[ct], window, chunked) : 0;
+    else start[ct] = (live && window > 0 && pos[ct] - window + 1 > 0) ? pos[ct] - window + 1 : 0;
   }
   bf16x8 qf[CT][HD / 32];  // B operands of the first product: column tile ct, features 32 j ..
 #pragma unroll
@@ -296,8 +319,10 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_split_kernel(
     for (int j = 0; j < HD / 32; ++j) qf[ct][j] = *reinterpret_cast<const bf16x8*>(qrow + 32 * j + 8 * g4);
   }
   const int hi = pos0 + ntok - 1;                                                        // last key any token sees
-  const int lo = (window > 0 && pos0 - window + 1 > 0) ? (pos0 - window + 1) / UNIT * UNIT : 0;  // first, rounded down
-  const int last_start = (window > 0 && hi - window + 1 > 0) ? hi - window + 1 : 0;     // window start of the last token
+  const int lo = BIASED ? first_visible(pos0, window, chunked) / UNIT * UNIT
+                        : ((window > 0 && pos0 - window + 1 > 0) ? (pos0 - window + 1) / UNIT * UNIT : 0);  // first, rounded down
+  const int last_start = BIASED ? first_visible(hi, window, chunked)
+                                : ((window > 0 && hi - window + 1 > 0) ? hi - window + 1 : 0);  // window start of the last token
 
   f32x4 acc[CT][HD / 16];  // O^T: rows hd = 16 t + 4 g4 + i, column = lane % 16
   float ref[CT], l[CT];    // the column's reference (log2 units) and this lane's share of its sum of weights
@@ -388,6 +413,15 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_split_kernel(
         for (int p = 0; p < 2; ++p)
 #pragma unroll
           for (int i = 0; i < 4; ++i) s[ct][p][i] = cap_over_scale * tanh_fast(s[ct][p][i] * scale_over_cap);
+    }
+    if (BIASED && slope_over_scale != 0.f) {  // s <- s - (slope / scale) (position - key): the scale follows as before
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+        for (int p = 0; p < 2; ++p)
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            s[ct][p][i] -= slope_over_scale * (float)(pos[ct] - (key0 + 16 * p + 4 * g4 + i));
     }
     if (more) load_keys(key0 + 4 * UNIT);  // into the registers the first product has just read
     if (!(key0 + UNIT - 1 <= pos0 && key0 >= last_start)) {  // some key is hidden from some token of the run
@@ -505,6 +539,7 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_split_kernel(
       if (c < ntok) {
         const float inv = 1.0f / sum;
         bf16_t* o = out + (int64_t)(tok0 + c) * out_stride + (int64_t)head * HD;
+        const bf16_t* gt = (BIASED && gate) ? gate + (int64_t)(tok0 + c) * gate_stride + (int64_t)head * HD + 4 * g4 : nullptr;
 #pragma unroll
         for (int t = 0; t < HD / 16; ++t) {
           s16x4 w4;
@@ -513,7 +548,9 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_split_kernel(
             float a = acc[ct][t][i] * own;
 #pragma unroll
             for (int w = 0; w < 3; ++w) a += s_acc[w][t][i][lane] * scale_w[w];
-            w4[i] = bf16_bits(a * inv);
+            a *= inv;
+            if (BIASED && gt) a /= 1.0f + expf(-__bfloat162float(gt[16 * t + i]));
+            w4[i] = bf16_bits(a);
           }
           *reinterpret_cast<s16x4*>(o + 16 * t + 4 * g4) = w4;
         }
@@ -556,11 +593,15 @@ extern "C" int pae_attn_decode_split() { return 64 * DECODE_TPW; }
 // max_splits = ceil(max_blocks * bs / pae_attn_decode_split()).
 // `cap` > 0: scores are capped, s <- cap tanh(s / cap); `sinks` (float32 [nh], or null): one number per query
 // head that joins its softmax's denominator as exp(sink).
-extern "C" int pae_attn_decode_capped_bf16(void* out, int64_t out_stride, const void* q, int64_t q_stride,
+static int attn_decode_any(void* out, int64_t out_stride, const void* q, int64_t q_stride,
                                     const void* k_cache, const void* v_cache, const int* dec_work, int num_dec,
                                     const int* block_tables, int max_blocks, int bs, int nh, int nkv, int hd, float scale, int window,
-                                    float cap, const float* sinks, void* part_acc, void* part_ml, hipStream_t stream) {
+                                    float cap, const float* sinks, void* part_acc, void* part_ml, bool biased, int chunked,
+                                    const float* slopes, const void* gate, int64_t gate_stride, hipStream_t stream) {
   if (int rc = check_common("attn_decode", nh, nkv, hd, bs, max_blocks, window)) return rc;
+  PAE_REQUIRE(!biased || cap == 0.f, "attn_decode: a bias by distance and a score cap together are not built");
+  PAE_REQUIRE(biased || (!chunked && !slopes && !gate), "attn_decode: chunks, slopes and gates belong to the biased kernels");
+  PAE_REQUIRE(!gate || gate_stride >= (int64_t)nh * hd, "attn_decode: gate row stride %lld too small", (long long)gate_stride);
   PAE_REQUIRE(num_dec <= 65535 && nkv <= 65535, "attn_decode: grid too large");
   if (num_dec <= 0) return 0;
   const int split_len = 64 * DECODE_TPW;
@@ -578,24 +619,46 @@ extern "C" int pae_attn_decode_capped_bf16(void* out, int64_t out_stride, const 
   const size_t merge_lds = (size_t)(merge_groups - 1) * merge_items * 6 * sizeof(float);
   PAE_REQUIRE(cap >= 0.f, "attn_decode: negative score cap %g", (double)cap);
   const float cap_log2 = cap * LOG2E, scale_over_cap = cap > 0.f ? scale / cap : 0.f;
-#define CALL_CAPPED(HD, CAPPED)                                                                              \
-  attn_decode_kernel<HD, DECODE_TPW, CAPPED><<<grid, 256, (size_t)3 * (HD / 4 + 2) * PAE_WAVE * sizeof(float), stream>>>( \
+#define CALL_CAPPED(HD, CAPPED, BIASED)                                                                      \
+  attn_decode_kernel<HD, DECODE_TPW, CAPPED, BIASED><<<grid, 256, (size_t)3 * (HD / 4 + 2) * PAE_WAVE * sizeof(float), stream>>>( \
       (float*)part_acc, (float*)part_ml, max_splits, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache,     \
       (const bf16_t*)v_cache, (const int4*)dec_work, block_tables, max_blocks, bs, nh, nkv, scale_log2, \
-      window, cap_log2, scale_over_cap)
+      window, cap_log2, scale_over_cap, chunked, slopes)
 #define CALL(HD)                                                                                            \
-  if (cap > 0.f) {                                                                                          \
-    CALL_CAPPED(HD, true);                                                                                  \
+  if (biased) {                                                                                             \
+    CALL_CAPPED(HD, false, true);                                                                           \
+  } else if (cap > 0.f) {                                                                                   \
+    CALL_CAPPED(HD, true, false);                                                                           \
   } else {                                                                                                  \
-    CALL_CAPPED(HD, false);                                                                                 \
+    CALL_CAPPED(HD, false, false);                                                                          \
   }                                                                                                         \
   attn_decode_merge_kernel<HD, DECODE_TPW><<<merge_grid, dim3(merge_x, merge_groups), merge_lds, stream>>>( \
       (bf16_t*)out, out_stride, (const float*)part_acc, (const float*)part_ml, max_splits, (const int4*)dec_work, \
-      nh, nkv, window, sinks)
+      nh, nkv, window, sinks, chunked, (const bf16_t*)gate, gate_stride)
   FOR_HEAD_DIM(hd, CALL)
 #undef CALL
 #undef CALL_CAPPED
   return pae_check_launch("attn_decode");
+}
+
+extern "C" int pae_attn_decode_capped_bf16(void* out, int64_t out_stride, const void* q, int64_t q_stride,
+                                    const void* k_cache, const void* v_cache, const int* dec_work, int num_dec,
+                                    const int* block_tables, int max_blocks, int bs, int nh, int nkv, int hd, float scale, int window,
+                                    float cap, const float* sinks, void* part_acc, void* part_ml, hipStream_t stream) {
+  return attn_decode_any(out, out_stride, q, q_stride, k_cache, v_cache, dec_work, num_dec, block_tables, max_blocks, bs, nh,
+                         nkv, hd, scale, window, cap, sinks, part_acc, part_ml, false, 0, nullptr, nullptr, 0, stream);
+}
+
+// `chunked`: the window is a chunk length; `slopes` (float32 [nh] or null): score -= slopes[h] (position - key);
+// `gate` (bfloat16 rows [token][nh * hd], or null): out *= sigmoid(gate).
+extern "C" int pae_attn_decode_biased_bf16(void* out, int64_t out_stride, const void* q, int64_t q_stride,
+                                    const void* k_cache, const void* v_cache, const int* dec_work, int num_dec,
+                                    const int* block_tables, int max_blocks, int bs, int nh, int nkv, int hd, float scale, int window,
+                                    int chunked, const float* slopes, const void* gate, int64_t gate_stride, void* part_acc,
+                                    void* part_ml, hipStream_t stream) {
+  return attn_decode_any(out, out_stride, q, q_stride, k_cache, v_cache, dec_work, num_dec, block_tables, max_blocks, bs, nh,
+                         nkv, hd, scale, window, 0.f, nullptr, part_acc, part_ml, true, chunked, slopes, gate, gate_stride,
+                         stream);
 }
 
 extern "C" int pae_attn_decode_bf16(void* out, int64_t out_stride, const void* q, int64_t q_stride,
@@ -608,12 +671,17 @@ extern "C" int pae_attn_decode_bf16(void* out, int64_t out_stride, const void* q
 
 // tiles[t] = (table row of the sequence, first flat token, number of tokens <= 64), heaviest runs
 // first: workgroups start in the order of the grid, and the last to finish sets the time.
-extern "C" int pae_attn_prefill_capped_bf16(void* out, int64_t out_stride, const void* q, int64_t q_stride,
+static int attn_prefill_any(void* out, int64_t out_stride, const void* q, int64_t q_stride,
                                           const void* k_cache, const void* v_cache, const int* tiles,
                                           int num_tiles, const int* positions, const int* block_tables,
                                           int max_blocks, int bs, int nh, int nkv, int hd, float scale, int window,
-                                          float cap, const float* sinks, hipStream_t stream) {
+                                          float cap, const float* sinks, bool biased, int chunked, const float* slopes,
+                                          const void* gate, int64_t gate_stride, hipStream_t stream) {
   if (int rc = check_common("attn_prefill", nh, nkv, hd, bs, max_blocks, window)) return rc;
+  PAE_REQUIRE(!biased || cap == 0.f, "attn_prefill: a bias by distance and a score cap together are not built");
+  PAE_REQUIRE(!biased || !slopes || scale > 0.f, "attn_prefill: a bias by distance needs a positive scale");
+  PAE_REQUIRE(biased || (!chunked && !slopes && !gate), "attn_prefill: chunks, slopes and gates belong to the biased kernels");
+  PAE_REQUIRE(!gate || gate_stride >= (int64_t)nh * hd, "attn_prefill: gate row stride %lld too small", (long long)gate_stride);
   PAE_REQUIRE(num_tiles <= 65535, "attn_prefill: %d runs exceed the grid", num_tiles);
   if (num_tiles <= 0) return 0;
   const float scale_log2 = scale * LOG2E;
@@ -624,16 +692,18 @@ extern "C" int pae_attn_prefill_capped_bf16(void* out, int64_t out_stride, const
   const bool halves = (int64_t)nh * num_tiles <= 256;
   PAE_REQUIRE(cap >= 0.f && (cap == 0.f || scale > 0.f), "attn_prefill: bad score cap %g (scale %g)", (double)cap, (double)scale);
   const float cap_over_scale = cap > 0.f ? cap / scale : 0.f, scale_over_cap = cap > 0.f ? scale / cap : 0.f;
-#define LAUNCH_CAPPED(HD, CT, BS, CAPPED)                                                                      \
-  attn_prefill_split_kernel<HD, CT, BS, CAPPED><<<dim3(nh, num_tiles, 4 / CT), 256, 0, stream>>>(              \
+#define LAUNCH_CAPPED(HD, CT, BS, CAPPED, BIASED)                                                              \
+  attn_prefill_split_kernel<HD, CT, BS, CAPPED, BIASED><<<dim3(nh, num_tiles, 4 / CT), 256, 0, stream>>>(      \
       (bf16_t*)out, out_stride, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache,    \
       tiles, positions, block_tables, max_blocks, bs, nh, nkv, scale_log2, window, cap_over_scale,             \
-      scale_over_cap, sinks)
-#define LAUNCH_CT(HD, CT, BS)           \
-  if (cap > 0.f) {                      \
-    LAUNCH_CAPPED(HD, CT, BS, true);    \
-  } else {                              \
-    LAUNCH_CAPPED(HD, CT, BS, false);   \
+      scale_over_cap, sinks, chunked, slopes, slopes ? 1.0f / scale : 0.f, (const bf16_t*)gate, gate_stride)
+#define LAUNCH_CT(HD, CT, BS)                  \
+  if (biased) {                                \
+    LAUNCH_CAPPED(HD, CT, BS, false, true);    \
+  } else if (cap > 0.f) {                      \
+    LAUNCH_CAPPED(HD, CT, BS, true, false);    \
+  } else {                                     \
+    LAUNCH_CAPPED(HD, CT, BS, false, false);   \
   }
 #define LAUNCH(HD, BS)                  \
   if (HD > 128 || halves) {             \
@@ -653,6 +723,26 @@ extern "C" int pae_attn_prefill_capped_bf16(void* out, int64_t out_stride, const
 #undef LAUNCH_CT
 #undef LAUNCH_CAPPED
   return pae_check_launch("attn_prefill");
+}
+
+extern "C" int pae_attn_prefill_capped_bf16(void* out, int64_t out_stride, const void* q, int64_t q_stride,
+                                          const void* k_cache, const void* v_cache, const int* tiles,
+                                          int num_tiles, const int* positions, const int* block_tables,
+                                          int max_blocks, int bs, int nh, int nkv, int hd, float scale, int window,
+                                          float cap, const float* sinks, hipStream_t stream) {
+  return attn_prefill_any(out, out_stride, q, q_stride, k_cache, v_cache, tiles, num_tiles, positions, block_tables,
+                          max_blocks, bs, nh, nkv, hd, scale, window, cap, sinks, false, 0, nullptr, nullptr, 0, stream);
+}
+
+extern "C" int pae_attn_prefill_biased_bf16(void* out, int64_t out_stride, const void* q, int64_t q_stride,
+                                          const void* k_cache, const void* v_cache, const int* tiles,
+                                          int num_tiles, const int* positions, const int* block_tables,
+                                          int max_blocks, int bs, int nh, int nkv, int hd, float scale, int window,
+                                          int chunked, const float* slopes, const void* gate, int64_t gate_stride,
+                                          hipStream_t stream) {
+  return attn_prefill_any(out, out_stride, q, q_stride, k_cache, v_cache, tiles, num_tiles, positions, block_tables,
+                          max_blocks, bs, nh, nkv, hd, scale, window, 0.f, nullptr, true, chunked, slopes, gate, gate_stride,
+                          stream);
 }
 
 extern "C" int pae_attn_prefill_bf16(void* out, int64_t out_stride, const void* q, int64_t q_stride,

@@ -91,6 +91,8 @@ def _declare(lib) -> None:
         "pae_sample_static_prepare": [],
         "pae_attn_decode_bf16": [P, L, P, L, P, P, P, I, P, I, I, I, I, I, F, I, P, P, P],
         "pae_attn_decode_split": [],
+        "pae_attn_decode_biased_bf16": [P, L, P, L, P, P, P, I, P, I, I, I, I, I, F, I, I, P, P, L, P, P, P],
+        "pae_attn_prefill_biased_bf16": [P, L, P, L, P, P, P, I, P, P, I, I, I, I, I, F, I, I, P, P, L, P],
         "pae_attn_decode_capped_bf16": [P, L, P, L, P, P, P, I, P, I, I, I, I, I, F, I, F, P, P, P, P],
         "pae_attn_prefill_capped_bf16": [P, L, P, L, P, P, P, I, P, P, I, I, I, I, I, F, I, F, P, P],
         "pae_attn_prefill_bf16": [P, L, P, L, P, P, P, I, P, P, I, I, I, I, I, F, I, P],
@@ -1254,6 +1256,17 @@ def delta_rule_step(proj: torch.Tensor, out: torch.Tensor, tok_seq: torch.Tensor
         float(norm_eps), work.data_ptr(), out.data_ptr(), _stream()))
 
 
+def _check_bias_operands(slopes, gate, nh: int, hd: int, q: torch.Tensor):
+    """(gate pointer, gate row stride) after checking the slopes and the gate rows of a biased attention call."""
+    if slopes is not None:
+        assert slopes.dtype == torch.float32 and slopes.numel() == nh and slopes.is_contiguous()
+    if gate is None:
+        return None, 0
+    assert gate.dim() == 2 and gate.shape[0] == q.shape[0] and gate.stride(1) == 1 and gate.shape[1] >= nh * hd
+    assert gate.dtype == torch.bfloat16
+    return gate.data_ptr(), gate.stride(0)
+
+
 def mfma_attention_supported(dtype: torch.dtype, nh: int, nkv: int, hd: int, bs: int) -> bool:
     """Shapes the matrix-core attention kernels take; others go through the generic kernel."""
     return dtype == torch.bfloat16 and hd % 32 == 0 and 32 <= hd <= 256 and bs % 16 == 0 and nh // nkv <= 16
@@ -1261,13 +1274,17 @@ def mfma_attention_supported(dtype: torch.dtype, nh: int, nkv: int, hd: int, bs:
 
 def attn_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                 dec_work: torch.Tensor, block_tables: torch.Tensor, nh: int, nkv: int, hd: int, scale: float,
-                window: int, softcap: float = 0.0, sinks: Optional[torch.Tensor] = None) -> None:
+                window: int, softcap: float = 0.0, sinks: Optional[torch.Tensor] = None, chunked: bool = False,
+                slopes: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> None:
     """Attention of the single new token of each sequence listed in `dec_work` over that sequence's
     cached keys: split over the keys, then merged.  dec_work[i] = (flat row of the token, its
     position, row of its sequence in `block_tables`, 0).  `softcap` > 0 caps the scores
-    (s <- softcap tanh(s / softcap)); `sinks` (float32 [nh]) join each head's softmax denominator."""
-    _gpu(out, q, k_cache, v_cache, dec_work, block_tables, sinks)
+    (s <- softcap tanh(s / softcap)); `sinks` (float32 [nh]) join each head's softmax denominator.
+    `chunked`, `slopes`, `gate`: as in `paged_attention_masked` (not together with a cap or sinks)."""
+    _gpu(out, q, k_cache, v_cache, dec_work, block_tables, sinks, slopes, gate)
     wide = bool(softcap) or sinks is not None
+    biased = chunked or slopes is not None or gate is not None
+    assert not (wide and biased)
     if sinks is not None:
         assert sinks.dtype == torch.float32 and sinks.numel() == nh and sinks.is_contiguous()
     bs = k_cache.shape[2]
@@ -1283,6 +1300,14 @@ def attn_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cac
     max_splits = -(-block_tables.shape[1] * bs // library().pae_attn_decode_split())
     part_acc = torch.empty((n * nh * max_splits, hd), dtype=torch.float32, device=q.device)
     part_ml = torch.empty((n * nh * max_splits, 2), dtype=torch.float32, device=q.device)
+    if biased:
+        _not_while_recording("attn_decode with chunks, a bias by distance or a gate")
+        gp, gs = _check_bias_operands(slopes, gate, nh, hd, q)
+        _check(library().pae_attn_decode_biased_bf16(
+            out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
+            dec_work.data_ptr(), n, block_tables.data_ptr(), block_tables.shape[1], bs, nh, nkv, hd, float(scale),
+            int(window), 1 if chunked else 0, _ptr(slopes), gp, gs, part_acc.data_ptr(), part_ml.data_ptr(), _stream()))
+        return
     if wide:
         _not_while_recording("attn_decode with a score cap or sinks")
         _check(library().pae_attn_decode_capped_bf16(
@@ -1311,13 +1336,16 @@ PREFILL_TILE = 64  # tokens per run of the prefill attention kernel (one workgro
 def attn_prefill(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                  tiles: torch.Tensor, positions: torch.Tensor, block_tables: torch.Tensor,
                  nh: int, nkv: int, hd: int, scale: float, window: int, softcap: float = 0.0,
-                 sinks: Optional[torch.Tensor] = None) -> None:
+                 sinks: Optional[torch.Tensor] = None, chunked: bool = False, slopes: Optional[torch.Tensor] = None,
+                 gate: Optional[torch.Tensor] = None) -> None:
     """Attention of runs of consecutive tokens; tiles[t] = (table row of the sequence, first
     flat token, number of tokens <= PREFILL_TILE).  One workgroup per run and head, whose
     wavefronts share out the keys; workgroups start in the order of `tiles`, so the runs with
-    the most keys should come first.  `softcap` and `sinks` as in `attn_decode`."""
+    the most keys should come first.  `softcap`, `sinks`, `chunked`, `slopes` and `gate` as in `attn_decode`."""
     _not_while_recording("attn_prefill")
-    _gpu(out, q, k_cache, v_cache, tiles, positions, block_tables, sinks)
+    _gpu(out, q, k_cache, v_cache, tiles, positions, block_tables, sinks, slopes, gate)
+    biased = chunked or slopes is not None or gate is not None
+    assert not (biased and (softcap or sinks is not None))
     if sinks is not None:
         assert sinks.dtype == torch.float32 and sinks.numel() == nh and sinks.is_contiguous()
     bs = k_cache.shape[2]
@@ -1327,6 +1355,13 @@ def attn_prefill(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_ca
     assert tiles.dtype == torch.int32 and tiles.dim() == 2 and tiles.shape[1] == 3 and tiles.is_contiguous()
     assert positions.dtype == torch.int32 and positions.numel() == q.shape[0]
     assert block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous()
+    if biased:
+        gp, gs = _check_bias_operands(slopes, gate, nh, hd, q)
+        _check(library().pae_attn_prefill_biased_bf16(
+            out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
+            tiles.data_ptr(), tiles.shape[0], positions.data_ptr(), block_tables.data_ptr(), block_tables.shape[1],
+            bs, nh, nkv, hd, float(scale), int(window), 1 if chunked else 0, _ptr(slopes), gp, gs, _stream()))
+        return
     _check(library().pae_attn_prefill_capped_bf16(
         out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
         tiles.data_ptr(), tiles.shape[0], positions.data_ptr(), block_tables.data_ptr(), block_tables.shape[1],

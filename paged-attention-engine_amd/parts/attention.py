@@ -339,9 +339,17 @@ class PagedAttention(Part):
             first = self.conv_channels
             gate = proj[:, first:first + s.num_heads * s.v_dim]
         attn = torch.empty((proj.shape[0], s.num_heads * s.v_dim), dtype=proj.dtype, device=proj.device)
-        K.paged_attention_masked(attn, q, pages["k"], pages["v"], ctx.positions, ctx.tok_seq, table, s.num_heads,
-                                 s.num_kv_heads, s.head_dim, s.v_dim, s.scale, s.window or 0, s.mask == "chunk",
-                                 self.slopes, gate)
+        chunked = s.mask == "chunk"
+        if self._matrix_cores(ctx.cache.block_size) and s.scale > 0:
+            # single tokens by the decode kernel, runs of tokens by the prefill kernel, both on the matrix cores
+            geometry = (s.num_heads, s.num_kv_heads, s.head_dim, s.scale, s.window or 0, 0.0, None, chunked, self.slopes, gate)
+            if lists["decode_work"].numel():
+                K.attn_decode(attn, q, pages["k"], pages["v"], lists["decode_work"], table, *geometry)
+            if lists["prefill_tiles"].numel():
+                K.attn_prefill(attn, q, pages["k"], pages["v"], lists["prefill_tiles"], ctx.positions, table, *geometry)
+        else:
+            K.paged_attention_masked(attn, q, pages["k"], pages["v"], ctx.positions, ctx.tok_seq, table, s.num_heads,
+                                     s.num_kv_heads, s.head_dim, s.v_dim, s.scale, s.window or 0, chunked, self.slopes, gate)
         return self.out.branch(attn, ctx.sink)
 
     def forward(self, ctx, x):
