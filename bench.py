@@ -77,18 +77,52 @@ def danonex_shape(shape: dict, layers: int) -> dict:
             "layers": [recurrent if i % 4 == 1 else attention for i in range(layers)]}
 
 
+def ritalorn_shape(shape: dict, layers: int) -> dict:
+    """A Ritalorn configuration with the layer sizes of the Qwen2.5 shape `shape`: the same width, head counts
+    and head size in its attention layers (values as wide as keys, convolutions of four taps, chunks of 8,192
+    tokens), latent attention in every fourth layer (as many heads, the head size unrotated plus half of it
+    rotated, a latent of four head sizes, a window of 4,096), the second attention layer after each latent
+    one reading the first one's keys and values, the same feed-forward width (gated), the same vocabulary,
+    four copies of the stream."""
+    heads, kv, hd = shape["num_attention_heads"], shape["num_key_value_heads"], shape["head_dim"]
+    mlp = {"kind": "dense", "ff": shape["intermediate_size"]}
+
+    def attention(kv_from=None):
+        mixer = {"heads": heads, "kv_heads": kv, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "conv": 4, "mask": {"size": 8192}}
+        if kv_from is not None:
+            mixer["kv_from"] = kv_from
+        return {"type": "attention", "mlp": mlp, "mixer": mixer}
+
+    latent = {"type": "latent_attention", "mlp": mlp,
+              "mixer": {"heads": heads, "dim": hd, "rot_dim": hd // 2, "vdim": hd, "kv_rank": 4 * hd,
+                        "scale": (hd + hd // 2) ** -0.5, "rot": {"base": float(shape["rope_theta"]), "dims": hd // 2},
+                        "mask": {"size": 4096}}}
+    out = []
+    for i in range(layers):
+        out.append(latent if i % 4 == 1 else attention(i - 3 if i % 4 == 3 else None))
+    return {"architecture": "Ritalorn", "vocab": shape["vocab_size"], "width": shape["hidden_size"],
+            "norm": {"eps": shape["rms_norm_eps"]}, "streams": 4, "logit_softcap": 30.0, "layers": out}
+
+
 def design_run(args, shape: dict) -> int:
-    """`--design danonex`: decode steps (batch 1, 8, 64 at the context asked for) and a 2,048-token
-    prefill of a Danonex model with the shape's layer sizes, and beside each the same measurement of the
-    Qwen2.5 shape with the same number of layers.  One JSON line."""
+    """`--design danonex|ritalorn`: decode steps (batch 1, 8, 64 at the context asked for) and prefills of
+    2,048 and 8,192 tokens of a model of that design with the shape's layer sizes, and beside each the same
+    measurement of the Qwen2.5 shape (and, for ritalorn, of the Danonex shape) with the same number of
+    layers.  One JSON line."""
     import torch
 
     layers = args.layers or 8
-    record = {"metric": f"Danonex beside Qwen2.5 at the {args.model} layer sizes, {layers} layers: decode tok/s and "
+    title = args.design.capitalize()
+    record = {"metric": f"{title} beside Qwen2.5 at the {args.model} layer sizes, {layers} layers: decode tok/s and "
                         f"prefill tok/s", "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
               "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "context": args.ctx,
               "data": "synthetic: seeded uniform token ids, random weights N(0, 0.02)", "designs": {}}
-    configs = {"danonex": danonex_shape(shape, layers), "qwen2": dict(shape, num_hidden_layers=layers)}
+    if args.design == "ritalorn":
+        configs = {"ritalorn": ritalorn_shape(shape, layers)}
+        if not args.alone:
+            configs.update({"danonex": danonex_shape(shape, layers), "qwen2": dict(shape, num_hidden_layers=layers)})
+    else:
+        configs = {"danonex": danonex_shape(shape, layers), "qwen2": dict(shape, num_hidden_layers=layers)}
     for name, cfg in configs.items():
         model = build_model(cfg, args.dtype)
         vocab_cfg = {"vocab_size": shape["vocab_size"], "max_position_embeddings": shape.get("max_position_embeddings")}
@@ -104,7 +138,7 @@ def design_run(args, shape: dict) -> int:
         record["designs"][name] = out
         del model
         torch.cuda.empty_cache()
-    record["value"] = record["designs"]["danonex"]["decode_b8"]["tokens_per_s"]
+    record["value"] = record["designs"][args.design]["decode_b8"]["tokens_per_s"]
     print(json.dumps(record))
     return 0
 
@@ -337,10 +371,11 @@ def main() -> int:
     parser.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill runs")
     parser.add_argument("--prefill-only", action="store_true", help="time the 2,048-token prefill alone (for profiles)")
-    parser.add_argument("--design", choices=("qwen2", "danonex"), default="qwen2",
-                        help="danonex: a Danonex model with the shape's layer sizes (8 layers unless --layers says "
-                             "otherwise) beside the Qwen2.5 shape with as many layers: decode at batch 1, 8, 64 and "
-                             "prefills of 2,048 and 8,192 tokens")
+    parser.add_argument("--design", choices=("qwen2", "danonex", "ritalorn"), default="qwen2",
+                        help="danonex, ritalorn: a model of that design with the shape's layer sizes (8 layers unless "
+                             "--layers says otherwise) beside the Qwen2.5 shape (ritalorn: and the Danonex shape) with "
+                             "as many layers: decode at batch 1, 8, 64 and prefills of 2,048 and 8,192 tokens")
+    parser.add_argument("--alone", action="store_true", help="with --design ritalorn: that design only (for profiles)")
     args = parser.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU only: this engine has no multi-GPU path (run with --gpus 1)")
@@ -351,7 +386,7 @@ def main() -> int:
         print("bench.py needs a GPU", file=sys.stderr)
         return 1
     shape = QWEN25_1P5B if args.model == "1.5b" else OTHER_SHAPES[args.model]
-    if args.design == "danonex":
+    if args.design in ("danonex", "ritalorn"):
         try:
             return design_run(args, shape)
         except (Refused, Unresolved) as err:

@@ -85,7 +85,14 @@ int pae_conv_norm_store(int dtype, const void* proj, int64_t row_stride, void* q
 int pae_latent_prepare(int dtype, const void* proj, int64_t row_stride, void* q_full, int64_t qf_stride, int num_tokens,
                        int nh, int nope, int rd, int rot, int interleaved, int rank, const void* norm_w, int w_is_f32,
                        float eps, const float* cos_sin, const int* positions, const int* tok_seq, const int* block_tables,
-                       int max_blocks, int bs, void* latent, hipStream_t stream);
+                       int max_blocks, int bs, void* latent, void* latent_t, hipStream_t stream);
+// latent attention on the matrix cores: see attention_latent.hip
+int pae_latent_attn_supported(int kd, int C, int bs);
+int pae_latent_attn_columns(int H, int ct);
+int pae_latent_attn_bf16(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* latent,
+                         const void* latent_t, const int* tiles, int num_tiles, int ct, const int* positions,
+                         const int* block_tables, int max_blocks, int bs, int H, int kd, int C, float scale, int window,
+                         int chunked, hipStream_t stream);
 // rows [q | k | v]: whole-projection RMS norm of q and of k (weights null: none), rotation, cache write
 int pae_qk_norm_rotate_store(int dtype, void* qkv, int64_t row_stride, int num_tokens, int nh, int nkv, int hd, int vd,
                              const void* q_w, const void* k_w, int w_is_f32, float eps, int rot, int interleaved,

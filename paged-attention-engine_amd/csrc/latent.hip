@@ -5,7 +5,8 @@
 // workgroup per token:
 //   * divides the first kv_rank features of `down` by their root mean square (eps inside the root),
 //     multiplies by the norm's weight and writes them to the token's place in the latent pages,
-//     [block][offset][kv_rank + rd], features 0 .. kv_rank - 1;
+//     [block][offset][kv_rank + rd], features 0 .. kv_rank - 1 (and, if the caller keeps them, to the
+//     pages of transposed latents, [block][kv_rank][offset]);
 //   * rotates the first `rot` of the last rd features of `down` by the token's angles, pairs
 //     (2i, 2i + 1) if `interleaved` else (i, i + rot / 2), and writes all rd behind the latent;
 //   * rotates the last rd features of every query head likewise and writes them to
@@ -23,7 +24,7 @@ __global__ __launch_bounds__(256) void latent_prepare_kernel(
     const T* __restrict__ proj, int64_t row_stride, T* __restrict__ q_full, int64_t qf_stride, int nh, int nope, int rd,
     int rot, int interleaved, int rank, const void* __restrict__ norm_w, int w_is_f32, float eps,
     const float* __restrict__ cos_sin, const int* __restrict__ positions, const int* __restrict__ tok_seq,
-    const int* __restrict__ block_tables, int max_blocks, int bs, T* __restrict__ latent) {
+    const int* __restrict__ block_tables, int max_blocks, int bs, T* __restrict__ latent, T* __restrict__ latent_t) {
   __shared__ float scratch[4];
   const int t = blockIdx.x;
   const T* row = proj + (int64_t)t * row_stride;
@@ -35,8 +36,12 @@ __global__ __launch_bounds__(256) void latent_prepare_kernel(
   for (int i = threadIdx.x; i < rank; i += 256) { const float x = to_f32(down[i]); ss = fmaf(x, x, ss); }
   ss = block_sum<4>(ss, scratch);
   const float inv = 1.0f / sqrtf(ss / (float)rank + eps);
-  for (int i = threadIdx.x; i < rank; i += 256)
-    cached[i] = from_f32<T>(to_f32(down[i]) * inv * load_param(norm_w, w_is_f32, i));
+  for (int i = threadIdx.x; i < rank; i += 256) {
+    const T c = from_f32<T>(to_f32(down[i]) * inv * load_param(norm_w, w_is_f32, i));
+    cached[i] = c;
+    // the same latent transposed within the page, [block][rank][offset], for kernels that read values that way
+    if (latent_t) latent_t[(block * rank + i) * bs + pos % bs] = c;
+  }
   // rotated parts: "head" nh is the shared key part, heads 0 .. nh - 1 the queries'
   const int half = rot / 2;
   for (int idx = threadIdx.x; idx < (nh + 1) * half; idx += 256) {
@@ -62,7 +67,7 @@ extern "C" int pae_latent_prepare(int dtype, const void* proj, int64_t row_strid
                                   int num_tokens, int nh, int nope, int rd, int rot, int interleaved, int rank,
                                   const void* norm_w, int w_is_f32, float eps, const float* cos_sin, const int* positions,
                                   const int* tok_seq, const int* block_tables, int max_blocks, int bs, void* latent,
-                                  hipStream_t stream) {
+                                  void* latent_t, hipStream_t stream) {
   PAE_REQUIRE(nh > 0 && nope > 0 && rd >= 0 && rank > 0, "latent_prepare: bad sizes nh=%d nope=%d rd=%d rank=%d", nh, nope, rd,
               rank);
   PAE_REQUIRE(rot >= 0 && rot <= rd && rot % 2 == 0, "latent_prepare: %d rotated features of %d", rot, rd);
@@ -76,11 +81,11 @@ extern "C" int pae_latent_prepare(int dtype, const void* proj, int64_t row_strid
   if (dtype == PAE_F32)
     latent_prepare_kernel<float><<<num_tokens, 256, 0, stream>>>(
         (const float*)proj, row_stride, (float*)q_full, qf_stride, nh, nope, rd, rot, interleaved, rank, norm_w, w_is_f32, eps,
-        cos_sin, positions, tok_seq, block_tables, max_blocks, bs, (float*)latent);
+        cos_sin, positions, tok_seq, block_tables, max_blocks, bs, (float*)latent, (float*)latent_t);
   else if (dtype == PAE_BF16)
     latent_prepare_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>(
         (const bf16_t*)proj, row_stride, (bf16_t*)q_full, qf_stride, nh, nope, rd, rot, interleaved, rank, norm_w, w_is_f32,
-        eps, cos_sin, positions, tok_seq, block_tables, max_blocks, bs, (bf16_t*)latent);
+        eps, cos_sin, positions, tok_seq, block_tables, max_blocks, bs, (bf16_t*)latent, (bf16_t*)latent_t);
   else
     return pae_fail("latent_prepare: unknown dtype code %d", dtype);
   return pae_check_launch("latent_prepare");

@@ -77,7 +77,10 @@ def _declare(lib) -> None:
         "pae_hyper_spread": [P, P, I, I, I, P],
         "pae_hyper_collapse": [P, P, I, I, I, P],
         "pae_conv_norm_store": [I, P, L, P, L, I, I, P, P, P, P, P, P, L, I, I, I, I, I, I, F, P, I, I, P, P, P],
-        "pae_latent_prepare": [I, P, L, P, L, I, I, I, I, I, I, I, P, I, F, P, P, P, P, I, I, P, P],
+        "pae_latent_prepare": [I, P, L, P, L, I, I, I, I, I, I, I, P, I, F, P, P, P, P, I, I, P, P, P],
+        "pae_latent_attn_supported": [I, I, I],
+        "pae_latent_attn_columns": [I, I],
+        "pae_latent_attn_bf16": [P, L, P, L, P, P, P, I, I, P, P, I, I, I, I, I, F, I, I, P],
         "pae_gated_act": [I, P, P, I, I, I, I, P],
         "pae_gemm_plain_batched": [I, I, P, L, L, P, L, L, P, L, P, I, I, I, I, I, P],
         "pae_rows_from_residual": [I, P, P, L, P],
@@ -1048,14 +1051,19 @@ def conv_norm_store(proj: torch.Tensor, q_out: torch.Tensor, tok_seq: torch.Tens
 
 def latent_prepare(proj: torch.Tensor, q_full: torch.Tensor, nh: int, nope: int, rd: int, rot: int, interleaved: bool,
                    rank: int, norm_w: torch.Tensor, eps: float, cos_sin: Optional[torch.Tensor], positions: torch.Tensor,
-                   tok_seq: torch.Tensor, block_tables: torch.Tensor, latent: torch.Tensor) -> None:
+                   tok_seq: torch.Tensor, block_tables: torch.Tensor, latent: torch.Tensor,
+                   latent_t: Optional[torch.Tensor] = None) -> None:
     """Rows `proj` [T, nh (nope + rd) + rank + rd] = [query heads | down projection]: the first `rank`
     features of the down projection are RMS-normed with `norm_w` and, with the last rd (their first
     `rot` rotated by `cos_sin`), written to the token's row of `latent` [block][bs][rank + rd]; the
     query heads' last rd features are rotated likewise into q_full[t, h, rank:] (`q_full`
-    [T, nh * (rank + rd)], whose first `rank` features per head the caller fills)."""
+    [T, nh * (rank + rd)], whose first `rank` features per head the caller fills).  With `latent_t`
+    [block][rank][bs] the normed latents are also written transposed within the page."""
     _not_while_recording("latent_prepare")
-    _gpu(proj, q_full, norm_w, cos_sin, positions, tok_seq, block_tables, latent)
+    _gpu(proj, q_full, norm_w, cos_sin, positions, tok_seq, block_tables, latent, latent_t)
+    if latent_t is not None:
+        assert tuple(latent_t.shape) == (latent.shape[0], rank, latent.shape[1]) and latent_t.is_contiguous()
+        assert latent_t.dtype == latent.dtype
     T = proj.shape[0]
     assert proj.dim() == 2 and proj.stride(1) == 1 and proj.shape[1] >= nh * (nope + rd) + rank + rd
     assert q_full.shape == (T, nh * (rank + rd)) and q_full.stride(1) == 1 and q_full.dtype == proj.dtype
@@ -1069,7 +1077,44 @@ def latent_prepare(proj: torch.Tensor, q_full: torch.Tensor, nh: int, nope: int,
     _check(library().pae_latent_prepare(
         code_of(proj.dtype), proj.data_ptr(), proj.stride(0), q_full.data_ptr(), q_full.stride(0), T, nh, nope, rd, rot,
         1 if interleaved else 0, rank, wp, wf, float(eps), _ptr(cos_sin) if rot else None, positions.data_ptr(),
-        tok_seq.data_ptr(), block_tables.data_ptr(), block_tables.shape[1], latent.shape[1], latent.data_ptr(), _stream()))
+        tok_seq.data_ptr(), block_tables.data_ptr(), block_tables.shape[1], latent.shape[1], latent.data_ptr(),
+        _ptr(latent_t), _stream()))
+
+
+def latent_attn_supported(dtype: torch.dtype, row_width: int, rank: int, block_size: int = 16) -> bool:
+    """Shapes the matrix-core latent attention takes; others go through the kernel for any shape."""
+    return dtype == torch.bfloat16 and bool(library().pae_latent_attn_supported(row_width, rank, block_size))
+
+
+def latent_attn_tokens(num_heads: int, column_tiles: int) -> int:
+    """Tokens one workgroup of the matrix-core latent attention takes with that many tiles of 16 columns."""
+    return library().pae_latent_attn_columns(num_heads, column_tiles)
+
+
+def latent_attn(out: torch.Tensor, q_full: torch.Tensor, latent: torch.Tensor, latent_t: torch.Tensor, tiles: torch.Tensor,
+                column_tiles: int, positions: torch.Tensor, block_tables: torch.Tensor, nh: int, rank: int, scale: float,
+                window: int = 0, chunked: bool = False) -> None:
+    """Latent attention on the matrix cores.  `q_full` [T, nh * KD] holds per head the query folded into
+    latent space and its rotated part; `latent` [block][bs][KD] and `latent_t` [block][rank][bs] are the
+    cached rows and their transposed latents; tiles[i] = (table row, first flat token, tokens, 0) with at
+    most `latent_attn_tokens(nh, column_tiles)` tokens; out[t, h * rank:(h + 1) * rank] receives the
+    weighted sums of the latents."""
+    _not_while_recording("latent_attn")
+    _gpu(out, q_full, latent, latent_t, tiles, positions, block_tables)
+    T = q_full.shape[0]
+    kd, bs = latent.shape[2], latent.shape[1]
+    assert q_full.dtype == torch.bfloat16 == out.dtype == latent.dtype == latent_t.dtype
+    assert q_full.stride(1) == 1 and out.stride(1) == 1 and q_full.shape[1] >= nh * kd and out.shape[1] >= nh * rank
+    assert out.shape[0] == T and latent.is_contiguous() and latent_t.is_contiguous()
+    assert tuple(latent_t.shape) == (latent.shape[0], rank, bs)
+    assert tiles.dtype == torch.int32 and tiles.dim() == 2 and tiles.shape[1] == 4 and tiles.is_contiguous()
+    assert tiles.data_ptr() % 16 == 0
+    assert positions.dtype == torch.int32 and positions.numel() == T
+    assert block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous()
+    _check(library().pae_latent_attn_bf16(
+        out.data_ptr(), out.stride(0), q_full.data_ptr(), q_full.stride(0), latent.data_ptr(), latent_t.data_ptr(),
+        tiles.data_ptr(), tiles.shape[0], column_tiles, positions.data_ptr(), block_tables.data_ptr(), block_tables.shape[1],
+        bs, nh, kd, rank, float(scale), int(window), 1 if chunked else 0, _stream()))
 
 
 def hyper_norm(streams: torch.Tensor, num_streams: int, y: Optional[torch.Tensor], layer_scale: Optional[torch.Tensor],

@@ -25,13 +25,31 @@ import torch
 
 from ..cache.manager import PAGE, PagedSpec, PagedTensor
 from ..kernels import lib as K
-from .base import POSITION_ENCODINGS, Part, ScaleShape, build_part, plain_rows, register_mixer
+from .base import POSITION_ENCODINGS, Part, ScaleShape, StepShape, build_part, plain_rows, register_mixer
 from .linear import Linear, rows_a_graph_may_hold
 
 
-def latent_pages(kv_rank: int, rope_dim: int, window=None) -> PagedSpec:
-    """One row per token: the latent vector, then the rotated key part."""
-    return PagedSpec((PagedTensor("latent", (PAGE, kv_rank + rope_dim)),), window)
+def latent_pages(kv_rank: int, rope_dim: int, window=None, transposed: bool = False) -> PagedSpec:
+    """One row per token: the latent vector, then the rotated key part.  `transposed`: also the latents
+    transposed within the page, [kv_rank][PAGE], the layout the matrix-core kernel reads its values in."""
+    tensors = (PagedTensor("latent", (PAGE, kv_rank + rope_dim)),)
+    if transposed:
+        tensors += (PagedTensor("latent_t", (kv_rank, PAGE)),)
+    return PagedSpec(tensors, window)
+
+
+def latent_tiles(shape: StepShape, single: int, runs: int):
+    """Work lists of the matrix-core kernel: (table row, first flat token, tokens, 0) for every sequence that
+    brings one token (`single`), and for the others in pieces of up to `runs` tokens, those with the most keys first."""
+    one, many = [], []
+    for row, (start, n, past) in enumerate(zip(shape.q_starts, shape.q_lens, shape.past_lens)):
+        if n == 1:
+            one += [row, start, 1, 0]
+        else:
+            for first in range(0, n, runs):
+                many.append((past + first, (row, start + first, min(runs, n - first), 0)))
+    many.sort(key=lambda piece: -piece[0])
+    return {"single": (one, 4), "runs": ([x for _, piece in many for x in piece], 4)}
 
 
 @register_mixer("latent_attention")
@@ -68,9 +86,24 @@ class LatentAttention(Part):
     def row_width(self) -> int:
         return self.spec.kv_rank + self.spec.rope_dim
 
+    @property
+    def matrix_cores(self) -> bool:
+        """Whether the attention runs on the matrix cores (then the pages also hold the latents transposed)."""
+        return K.latent_attn_supported(self.dtype, self.row_width, self.spec.kv_rank)
+
     def paged_spec(self):
         s = self.spec
-        return latent_pages(s.kv_rank, s.rope_dim, s.window if s.mask == "window" else None)
+        return latent_pages(s.kv_rank, s.rope_dim, s.window if s.mask == "window" else None, self.matrix_cores)
+
+    def step_lists_key(self, block_size: int):
+        if not (self.matrix_cores and block_size % 16 == 0):
+            return None
+        H = self.spec.num_heads
+        return ("latent attention tiles", K.latent_attn_tokens(H, 1), K.latent_attn_tokens(H, 2))
+
+    def step_lists(self, shape: StepShape):
+        H = self.spec.num_heads
+        return latent_tiles(shape, K.latent_attn_tokens(H, 1), K.latent_attn_tokens(H, 2))
 
     def tensors(self, prefix):
         s = self.spec
@@ -100,17 +133,26 @@ class LatentAttention(Part):
             raise ValueError("a latent attention layer keeps pages of its own")
         x = plain_rows(x)
         T, H, C, R, D, V = x.shape[0], s.num_heads, s.kv_rank, s.rope_dim, s.nope_dim, s.value_dim
-        latent = ctx.cache.pages_of(ctx.cache_entry)["latent"]
+        pages = ctx.cache.pages_of(ctx.cache_entry)
+        latent, latent_t = pages["latent"], pages.get("latent_t")
         table = ctx.block_tables[ctx.cache.group_of(ctx.cache_entry)]
         proj = self.proj(x)
         rot, cos_sin = self.position.rotary_table(ctx)
         q_full = torch.empty((T, H * (C + R)), dtype=proj.dtype, device=proj.device)
         K.latent_prepare(proj, q_full, H, D, R, rot, bool(getattr(self.position, "interleaved", False)), C,
-                         self.down_norm, s.norm_eps, cos_sin, ctx.positions, ctx.tok_seq, table, latent)
+                         self.down_norm, s.norm_eps, cos_sin, ctx.positions, ctx.tok_seq, table, latent, latent_t)
         K.heads_product(q_full.view(T, H, C + R)[:, :, :C], proj[:, :H * (D + R)].view(T, H, D + R)[:, :, :D], self.up_k_t)
         summed = torch.empty((T, H * C), dtype=proj.dtype, device=proj.device)
-        K.paged_attention_masked(summed, q_full, latent, None, ctx.positions, ctx.tok_seq, table, H, 1, C + R, C, s.scale,
-                                 s.window or 0, s.mask == "chunk")
+        key = self.step_lists_key(ctx.cache.block_size)
+        if key is not None:
+            tiles = ctx.memo[key]
+            for name, column_tiles in (("single", 1), ("runs", 2)):
+                if tiles[name].numel():
+                    K.latent_attn(summed, q_full, latent, latent_t, tiles[name], column_tiles, ctx.positions, table, H, C,
+                                  s.scale, s.window or 0, s.mask == "chunk")
+        else:
+            K.paged_attention_masked(summed, q_full, latent, None, ctx.positions, ctx.tok_seq, table, H, 1, C + R, C, s.scale,
+                                     s.window or 0, s.mask == "chunk")
         heads = torch.empty((T, H * V), dtype=proj.dtype, device=proj.device)
         K.heads_product(heads.view(T, H, V), summed.view(T, H, C), self.up_v)
         return self.out.branch(heads, ctx.sink)

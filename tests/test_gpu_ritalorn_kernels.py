@@ -248,7 +248,8 @@ def test_the_spelled_out_attention_and_the_one_by_matrices_agree():
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,D,R,V,C,dims,bs,T,size", [(3, 16, 8, 24, 40, 8, 16, 150, 20), (2, 24, 16, 8, 16, 8, 8, 100, 7),
                                                       (4, 32, 32, 32, 64, 32, 16, 330, 100), (1, 40, 24, 72, 72, 24, 16, 80, 0),
-                                                      (2, 8, 4, 12, 300, 4, 16, 70, 33)])
+                                                      (2, 8, 4, 12, 300, 4, 16, 70, 33), (5, 32, 64, 32, 512, 64, 16, 200, 60),
+                                                      (20, 16, 32, 16, 64, 32, 32, 90, 0), (12, 16, 32, 16, 128, 32, 16, 75, 17)])
 @pytest.mark.parametrize("new", ["prompt", "portion", "single"])
 def test_latent_attention_from_projected_rows_to_heads(dtype, H, D, R, V, C, dims, bs, T, size, new):
     """Projected rows through the latent norm, the rotation, the page write, the fold of the queries, the attention over
@@ -283,8 +284,10 @@ def test_latent_attention_from_projected_rows_to_heads(dtype, H, D, R, V, C, dim
         inv_freq = torch.tensor([base ** (-2.0 * i / dims) for i in range(dims // 2)], dtype=torch.float32, device=DEV)
         cos_sin = K.rope_table(positions, inv_freq)
         q_full = torch.zeros(T, H * (C + R), dtype=dtype, device=DEV)
+        cores = K.latent_attn_supported(dtype, C + R, C, bs)
+        latent_t = torch.zeros(table.numel() + 2, C, bs, dtype=dtype, device=DEV) if cores else None
         K.latent_prepare(proj, q_full, H, D, R, dims, True, C, w["p.dkv.norm"].to(dtype).to(DEV), eps, cos_sin, positions, tok_seq,
-                         tables, latent)
+                         tables, latent, latent_t)
         up_k_t = w["p.uk"].view(H, D, C).transpose(1, 2).contiguous().to(dtype).to(DEV)
         K.heads_product(q_full.view(T, H, C + R)[:, :, :C], proj[:, :H * (D + R)].view(T, H, D + R)[:, :, :D], up_k_t)
         n = T - new_from
@@ -293,6 +296,21 @@ def test_latent_attention_from_projected_rows_to_heads(dtype, H, D, R, V, C, dim
                                  C + R, C, scale, size or 0)
         heads = torch.empty(n, H * V, dtype=dtype, device=DEV)
         K.heads_product(heads.view(n, H, V), summed.view(n, H, C), w["p.uv"].view(H, V, C).to(dtype).to(DEV))
+        if cores:  # the same on the matrix cores: single tokens one column tile, runs two
+            from paged_attention_engine_amd.parts import StepShape
+            from paged_attention_engine_amd.parts.latent import latent_tiles
+
+            assert torch.equal(latent_t.transpose(1, 2)[table.long()], latent[table.long()][:, :, :C])
+            lists = latent_tiles(StepShape((0,), (0,), (n,), (new_from,), bs), K.latent_attn_tokens(H, 1), K.latent_attn_tokens(H, 2))
+            fast = torch.zeros(n, H * C, dtype=dtype, device=DEV)
+            for name, column_tiles in (("single", 1), ("runs", 2)):
+                flat, width = lists[name]
+                if flat:
+                    tiles = torch.tensor(flat, dtype=torch.int32, device=DEV).view(-1, width)
+                    K.latent_attn(fast, q_full[new_from:], latent, latent_t, tiles, column_tiles, positions[new_from:], tables, H, C,
+                                  scale, size or 0)
+            top = float(summed.float().abs().max())
+            assert float((fast.float() - summed.float()).abs().max()) <= 2.5e-2 * top, f"matrix cores, key {key}"
         err = float((heads.cpu().double() - want).abs().max())
         bound = (5e-5 if dtype == torch.float32 else 6e-2) * float(want.abs().max())  # scores of tens: a rounding of q or k is a few 1e-6 of a weight
         assert err <= bound, f"key {key} of {first_seen}..{last}: {err} > {bound}"
