@@ -72,17 +72,21 @@ __global__ __launch_bounds__(256, 1) void latent_attn_kernel(
   }
 
   const int lrow = lane / 4, lgrp = lane % 4;
-  for (int key0 = lo + 16 * wave; key0 <= hi; key0 += 64) {
+  // Two register sets of keys and values take turns: the next tile's loads are in flight while this tile's
+  // products run (a wavefront walks its tiles alone, with no other wavefront of its own to hide the wait).
+  bf16x8 kfa[KD / 32], kfb[KD / 32];
+  s16x4 vfa[VS / 16], vfb[VS / 16];
+  auto load = [&](bf16x8 (&kf)[KD / 32], s16x4 (&vf)[VS / 16], int key0) {
     const int64_t block = max(table[key0 / bs], 0);  // a page the window has passed: all its keys are masked
     const bf16_t* kp = latent + (block * bs + key0 % bs) * (int64_t)KD;
     const bf16_t* vp = latent_t + (block * C + (int64_t)slice * VS) * bs + key0 % bs;
-    bf16x8 kf[KD / 32];
-    s16x4 vf[VS / 16];
 #pragma unroll
     for (int j = 0; j < KD / 32; ++j) kf[j] = *reinterpret_cast<const bf16x8*>(kp + lrow * KD + 32 * j + 8 * lgrp);
 #pragma unroll
     for (int t = 0; t < VS / 16; ++t)
       vf[t] = *reinterpret_cast<const s16x4*>(vp + (int64_t)(16 * t + col) * bs + 4 * g4);
+  };
+  auto compute = [&](bf16x8 (&kf)[KD / 32], s16x4 (&vf)[VS / 16], int key0) {
     keys_to_mfma_order<KD>(kf);
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
@@ -115,6 +119,21 @@ __global__ __launch_bounds__(256, 1) void latent_attn_kernel(
         acc[ct][t] *= alpha;
         acc[ct][t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf[t], pb, acc[ct][t], 0, 0, 0);
       }
+    }
+  };
+  int key0 = lo + 16 * wave;  // the same in every lane of a wavefront: the branches on it are uniform
+  if (key0 <= hi) {
+    load(kfa, vfa, key0);
+    while (true) {
+      const bool more_b = key0 + 64 <= hi;
+      if (more_b) load(kfb, vfb, key0 + 64);
+      compute(kfa, vfa, key0);
+      if (!more_b) break;
+      const bool more_a = key0 + 128 <= hi;
+      if (more_a) load(kfa, vfa, key0 + 128);
+      compute(kfb, vfb, key0 + 64);
+      if (!more_a) break;
+      key0 += 128;
     }
   }
 

@@ -909,7 +909,13 @@ def gemm_plain_heads(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor) -> Non
 
 
 def heads_product(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor) -> None:
-    """out[:, h, :] = a[:, h, :] @ w[h]^T for every head h (shapes as for `gemm_plain_heads`)."""
+    """out[:, h, :] = a[:, h, :] @ w[h]^T for every head h (shapes as for `gemm_plain_heads`).  bfloat16 with
+    more rows than the few-row kernels take goes to the platform's batched matrix product, as the plain
+    products of that many rows do; everything else to this engine's own kernel."""
+    if a.dtype == torch.bfloat16 and a.shape[0] > SKINNY_MAX_ROWS and _RECORDING is None:
+        # [B, M, K] x [B, K, N] on strided views: no copy of the operands; the result is copied into the view
+        out.copy_(torch.bmm(a.transpose(0, 1), w.transpose(1, 2)).transpose(0, 1))
+        return
     gemm_plain_heads(out, a, w)
 
 
