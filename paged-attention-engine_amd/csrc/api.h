@@ -44,6 +44,8 @@ int pae_gemm_skinny(int epilogue, void* out, int64_t ldc, const void* A, int64_t
 int pae_gemm_skinny_act(void* out, int64_t ldc, const void* A, int64_t lda, const void* W, const void* bias,
                         int b_is_f32, int M, int N, int K, int splits, float* ticket_parts, int* ticket_counters,
                         int act, hipStream_t stream);
+int pae_gemm_skinny_gated(void* out, int64_t ldc, const void* A, int64_t lda, const void* W, int M, int N, int K, int splits,
+                          float* ticket_parts, int* ticket_counters, int act, hipStream_t stream);
 int pae_skinny_ticket_slots(int M, int N);
 int64_t pae_skinny_ticket_floats(int M, int N, int splits);
 int pae_gemm_skinny_rope(void* q_out, int64_t ldq, const void* A, int64_t lda, const void* W, const void* bias,

@@ -578,6 +578,17 @@ extern "C" int pae_gemm_skinny_act(void* out, int64_t ldc, const void* A, int64_
                        SkinnyTickets{ticket_parts, ticket_counters}, norm, stream);
 }
 
+// The gated product (EPI_SWIGLU's layout of W: blocks of 8 gate rows followed by their 8 up rows) with the gate's
+// activation by code: out[M, N / 2] = act(gate) * up on the float32 sums.
+extern "C" int pae_gemm_skinny_gated(void* out, int64_t ldc, const void* A, int64_t lda, const void* W, int M, int N, int K,
+                                     int splits, float* ticket_parts, int* ticket_counters, int act, hipStream_t stream) {
+  PAE_REQUIRE(act >= 0 && act <= 2, "gemm_skinny_gated: unknown activation %d", act);
+  PAE_REQUIRE(N % 16 == 0 && ldc % 4 == 0, "gemm_skinny_gated: gated epilogue needs N %% 16 == 0, got %d", N);
+  const SkinnyNorm norm{nullptr, 0, 0.f, nullptr, 0, nullptr, 0, act + 1, nullptr};
+  return launch_skinny(EPI_SWIGLU, out, ldc, A, lda, W, nullptr, 0, M, N, K, splits, 0, SkinnyRope{},
+                       SkinnyTickets{ticket_parts, ticket_counters}, norm, stream);
+}
+
 // Counters and scratch floats that `splits` k ranges of an [M, K] x [N, K]^T product need for their
 // tickets, whichever kernel takes the product (one counter per wavefront that ends with whole sums of
 // its own; its accumulators for every range).

@@ -386,7 +386,8 @@ __device__ __forceinline__ void skinny_epilogue(const f32x4 (&acc)[RT][MT], int 
         for (int i = 0; i < 4; ++i) {
           const float own = acc[rt][mt][i] * scale[mt];
           const float up = __shfl_xor(own, 32);  // in every lane (the same row of A, so the same scale)
-          v[i] = to_bf16_bits(own / (1.0f + expf(-own)) * up);
+          // the gate's activation: SiLU, or the one the caller named (1 + its code, see act_of)
+          v[i] = to_bf16_bits((norm.act ? act_of(own, norm.act - 1) : own / (1.0f + expf(-own))) * up);
         }
         if (g4 < 2 && j < N / 2)  // N counts gate and up rows
           put<THROUGH>(reinterpret_cast<s16x4*>((bf16_t*)out + (int64_t)m * ldc + j), v);

@@ -69,6 +69,7 @@ def _declare(lib) -> None:
         "pae_skinny_ticket_slots": [I, I],
         "pae_gemm_skinny_act": [P, L, P, L, P, P, I, I, I, I, I, P, P, I, P],
         "pae_gemm_plain": [I, I, P, L, P, L, P, P, I, I, I, I, P],
+        "pae_gemm_skinny_gated": [P, L, P, L, P, I, I, I, I, P, P, I, P],
         "pae_paged_attention_generic": [I, P, L, P, L, P, P, P, P, P, I, I, I, I, I, I, F, I, P],
         "pae_paged_attention_capped": [I, P, L, P, L, P, P, P, P, P, I, I, I, I, I, I, I, F, I, F, P, P],
         "pae_qk_norm_rotate_store": [I, P, L, I, I, I, I, I, P, P, I, F, I, I, P, F, P, P, P, I, I, P, P, I, P],
@@ -703,6 +704,21 @@ def gemm_skinny_act(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, kind: s
     parts, counters = _ticket_scratch(a.device, M, N, splits)
     _launch_ticketed(counters, lambda: library().pae_gemm_skinny_act(
         out.data_ptr(), out.stride(0), a.data_ptr(), a.stride(0), w.data_ptr(), bp, bf, M, N, K_, splits, _ptr(parts),
+        _ptr(counters), ACTIVATIONS[kind], _stream()))
+
+
+def gemm_skinny_gated(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, kind: str, splits: int = 1) -> None:
+    """out [M, N / 2] bfloat16 = act(gate) * up for at most 64 rows of `a`, where w [N, K] holds blocks of 8
+    gate rows followed by their 8 up rows (the layout of EPI_SWIGLU) and `kind` names the gate's activation."""
+    _not_while_recording("gemm_skinny_gated")
+    _gpu(out, a, w)
+    M, K_ = a.shape
+    N = w.shape[0]
+    assert skinny_supported(a, w) and w.shape == (N, K_) and w.is_contiguous() and out.is_contiguous()
+    assert N % 16 == 0 and out.shape == (M, N // 2) and out.dtype == torch.bfloat16 and kind in ACTIVATIONS
+    parts, counters = _ticket_scratch(a.device, M, N, splits)
+    _launch_ticketed(counters, lambda: library().pae_gemm_skinny_gated(
+        out.data_ptr(), out.stride(0), a.data_ptr(), a.stride(0), w.data_ptr(), M, N, K_, splits, _ptr(parts),
         _ptr(counters), ACTIVATIONS[kind], _stream()))
 
 

@@ -66,6 +66,10 @@ class SwiGLU(Part):
             splits = K.whole_sum_splits(2 * self.spec.intermediate_size, self.spec.hidden_size, x.shape[0])
             K.gemm_skinny(act, rows, self.gate_up.weight, None, K.EPI_SWIGLU, splits,
                           row_scale=x.row_scale if isinstance(x, OwedRows) else None)
+        elif self.block and x.shape[0] and K.skinny_supported(rows, self.gate_up.weight) and not isinstance(x, OwedRows):
+            # another activation: the same product and layout, the activation by name in its epilogue
+            splits = K.whole_sum_splits(2 * self.spec.intermediate_size, self.spec.hidden_size, x.shape[0])
+            K.gemm_skinny_gated(act, rows, self.gate_up.weight, self.spec.activation, splits)
         elif self.silu:
             K.swiglu(act, self.gate_up(plain_rows(x)), self.block)
         else:

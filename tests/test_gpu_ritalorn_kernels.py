@@ -82,6 +82,21 @@ def test_the_gate_with_the_tanh_gelu(dtype):
     assert abs(float(plain.gelu_tanh(torch.tensor(1.0, dtype=torch.float64))) - 0.8411919906082768) < 1e-12
 
 
+@pytest.mark.parametrize("rows", [1, 8, 40])
+def test_the_few_row_gated_product_with_the_tanh_gelu(rows):
+    """Gate and up rows alternate in blocks of 8 in the weight; the activation runs on the float32 sums."""
+    K = _K()
+    gen = torch.Generator().manual_seed(rows)
+    inter, hidden = 48, 64
+    a = randn(gen, rows, hidden).to(torch.bfloat16)
+    gate, up = randn(gen, inter, hidden, scale=0.3).to(torch.bfloat16), randn(gen, inter, hidden, scale=0.3).to(torch.bfloat16)
+    w = torch.stack([gate.view(inter // 8, 8, hidden), up.view(inter // 8, 8, hidden)], dim=1).reshape(2 * inter, hidden)
+    want = plain.gelu_tanh(a.double() @ gate.double().T) * (a.double() @ up.double().T)
+    out = torch.empty(rows, inter, dtype=torch.bfloat16, device=DEV)
+    K.gemm_skinny_gated(out, a.to(DEV), w.contiguous().to(DEV), "gelu_tanh")
+    assert float((out.cpu().double() - want).abs().max()) <= 1e-2 * float(want.abs().max())
+
+
 # ------------------------------------------------------------------ convolutions, head norms, cache write
 def scattered_table(num_pages: int, spare: int, seed: int):
     gen = torch.Generator().manual_seed(seed)
