@@ -94,7 +94,8 @@ int pae_latent_attn_columns(int H, int ct);
 int pae_latent_attn_bf16(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* latent,
                          const void* latent_t, const int* tiles, int num_tiles, int ct, const int* positions,
                          const int* block_tables, int max_blocks, int bs, int H, int kd, int C, float scale, int window,
-                         int chunked, hipStream_t stream);
+                         int chunked, float* part_acc, float* part_ml, hipStream_t stream);
+int pae_latent_attn_split();
 // rows [q | k | v]: whole-projection RMS norm of q and of k (weights null: none), rotation, cache write
 int pae_qk_norm_rotate_store(int dtype, void* qkv, int64_t row_stride, int num_tokens, int nh, int nkv, int hd, int vd,
                              const void* q_w, const void* k_w, int w_is_f32, float eps, int rot, int interleaved,

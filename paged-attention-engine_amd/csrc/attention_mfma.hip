@@ -414,14 +414,21 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_split_kernel(
 #pragma unroll
           for (int i = 0; i < 4; ++i) s[ct][p][i] = cap_over_scale * tanh_fast(s[ct][p][i] * scale_over_cap);
     }
-    if (BIASED && slope_over_scale != 0.f) {  // s <- s - (slope / scale) (position - key): the scale follows as before
+    if (BIASED && slope_over_scale != 0.f) {
+      // s <- s - (slope / scale) (position - key); the scale follows as before.  A softmax does not see what is
+      // the same for all keys of a column, so the run's first position stands for every column's own: the term is
+      // formed once for the column tiles together (no score cap and no sink here, with which that would not hold).
+      float bias[2][4];
+#pragma unroll
+      for (int p = 0; p < 2; ++p)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) bias[p][i] = slope_over_scale * (float)(key0 + 16 * p + 4 * g4 + i - pos0);
 #pragma unroll
       for (int ct = 0; ct < CT; ++ct)
 #pragma unroll
         for (int p = 0; p < 2; ++p)
 #pragma unroll
-          for (int i = 0; i < 4; ++i)
-            s[ct][p][i] -= slope_over_scale * (float)(pos[ct] - (key0 + 16 * p + 4 * g4 + i));
+          for (int i = 0; i < 4; ++i) s[ct][p][i] += bias[p][i];
     }
     if (more) load_keys(key0 + 4 * UNIT);  // into the registers the first product has just read
     if (!(key0 + UNIT - 1 <= pos0 && key0 >= last_start)) {  // some key is hidden from some token of the run

@@ -81,7 +81,8 @@ def _declare(lib) -> None:
         "pae_latent_prepare": [I, P, L, P, L, I, I, I, I, I, I, I, P, I, F, P, P, P, P, I, I, P, P, P],
         "pae_latent_attn_supported": [I, I, I],
         "pae_latent_attn_columns": [I, I],
-        "pae_latent_attn_bf16": [P, L, P, L, P, P, P, I, I, P, P, I, I, I, I, I, F, I, I, P],
+        "pae_latent_attn_bf16": [P, L, P, L, P, P, P, I, I, P, P, I, I, I, I, I, F, I, I, P, P, P],
+        "pae_latent_attn_split": [],
         "pae_gated_act": [I, P, P, I, I, I, I, P],
         "pae_gemm_plain_batched": [I, I, P, L, L, P, L, L, P, L, P, I, I, I, I, I, P],
         "pae_rows_from_residual": [I, P, P, L, P],
@@ -1133,10 +1134,16 @@ def latent_attn(out: torch.Tensor, q_full: torch.Tensor, latent: torch.Tensor, l
     assert tiles.data_ptr() % 16 == 0
     assert positions.dtype == torch.int32 and positions.numel() == T
     assert block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous()
+    part_acc = part_ml = None
+    splits = -(-block_tables.shape[1] * bs // library().pae_latent_attn_split())
+    if column_tiles == 1 and splits > 1:
+        # single tokens with tables beyond one split: the keys are shared out over workgroups and merged
+        part_acc = torch.empty((tiles.shape[0] * splits * nh, rank), dtype=torch.float32, device=out.device)
+        part_ml = torch.empty((tiles.shape[0] * splits * nh, 2), dtype=torch.float32, device=out.device)
     _check(library().pae_latent_attn_bf16(
         out.data_ptr(), out.stride(0), q_full.data_ptr(), q_full.stride(0), latent.data_ptr(), latent_t.data_ptr(),
         tiles.data_ptr(), tiles.shape[0], column_tiles, positions.data_ptr(), block_tables.data_ptr(), block_tables.shape[1],
-        bs, nh, kd, rank, float(scale), int(window), 1 if chunked else 0, _stream()))
+        bs, nh, kd, rank, float(scale), int(window), 1 if chunked else 0, _ptr(part_acc), _ptr(part_ml), _stream()))
 
 
 def hyper_norm(streams: torch.Tensor, num_streams: int, y: Optional[torch.Tensor], layer_scale: Optional[torch.Tensor],
