@@ -88,6 +88,8 @@ int pae_latent_prepare(int dtype, const void* proj, int64_t row_stride, void* q_
                        int nh, int nope, int rd, int rot, int interleaved, int rank, const void* norm_w, int w_is_f32,
                        float eps, const float* cos_sin, const int* positions, const int* tok_seq, const int* block_tables,
                        int max_blocks, int bs, void* latent, void* latent_t, hipStream_t stream);
+int pae_heads_product_few(void* out, int64_t ldc, int64_t head_c, const void* a, int64_t lda, int64_t head_a, const void* w,
+                          int M, int N, int K, int heads, hipStream_t stream);  // bfloat16, a few rows, one product per head
 // latent attention on the matrix cores: see attention_latent.hip
 int pae_latent_attn_supported(int kd, int C, int bs);
 int pae_latent_attn_columns(int H, int ct);

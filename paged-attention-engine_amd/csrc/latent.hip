@@ -90,3 +90,45 @@ extern "C" int pae_latent_prepare(int dtype, const void* proj, int64_t row_strid
     return pae_fail("latent_prepare: unknown dtype code %d", dtype);
   return pae_check_launch("latent_prepare");
 }
+
+// One small product per head for a few rows (single tokens and short portions):
+//   out[m][h][n] = sum_k a[m][h][k] * w[h][n][k],   bfloat16 in and out, float32 sums.
+// One wavefront per (head, output feature): its lanes share out k (lane, lane + 64, ..), every row's partial sums
+// meet by a butterfly, lane 0 writes.  The weights (a few megabytes for all heads) are read once; with at most 64 rows
+// the rows stay in cache.  It stands where the plain product's batched entry would take a workgroup of 64 x 64
+// outputs for 8 x 128 of them.
+#define HEADS_FEW_ROWS 8  // rows a pass keeps sums for
+__global__ __launch_bounds__(256) void heads_product_few_kernel(bf16_t* __restrict__ out, int64_t ldc, int64_t head_c,
+                                                                const bf16_t* __restrict__ a, int64_t lda, int64_t head_a,
+                                                                const bf16_t* __restrict__ w, int M, int N, int K) {
+  const int lane = threadIdx.x % PAE_WAVE, wave = threadIdx.x / PAE_WAVE;
+  const int n = blockIdx.x * 4 + wave, h = blockIdx.y;
+  if (n >= N) return;
+  const bf16_t* wr = w + ((int64_t)h * N + n) * K;
+  for (int m0 = 0; m0 < M; m0 += HEADS_FEW_ROWS) {
+    float sum[HEADS_FEW_ROWS];
+#pragma unroll
+    for (int r = 0; r < HEADS_FEW_ROWS; ++r) sum[r] = 0.f;
+    for (int k = lane; k < K; k += PAE_WAVE) {
+      const float wk = to_f32(wr[k]);
+#pragma unroll
+      for (int r = 0; r < HEADS_FEW_ROWS; ++r)
+        if (m0 + r < M) sum[r] = fmaf(to_f32(a[(int64_t)(m0 + r) * lda + h * head_a + k]), wk, sum[r]);
+    }
+#pragma unroll
+    for (int r = 0; r < HEADS_FEW_ROWS; ++r) {
+      const float total = wave_sum(sum[r]);
+      if (lane == 0 && m0 + r < M) out[(int64_t)(m0 + r) * ldc + h * head_c + n] = __float2bfloat16(total);
+    }
+  }
+}
+
+extern "C" int pae_heads_product_few(void* out, int64_t ldc, int64_t head_c, const void* a, int64_t lda, int64_t head_a,
+                                     const void* w, int M, int N, int K, int heads, hipStream_t stream) {
+  PAE_REQUIRE(M >= 0 && N > 0 && K > 0 && heads > 0 && heads <= 65535, "heads_product_few: bad sizes M=%d N=%d K=%d heads=%d", M, N,
+              K, heads);
+  if (M == 0) return 0;
+  heads_product_few_kernel<<<dim3((N + 3) / 4, heads), 256, 0, stream>>>((bf16_t*)out, ldc, head_c, (const bf16_t*)a, lda, head_a,
+                                                                       (const bf16_t*)w, M, N, K);
+  return pae_check_launch("heads_product_few");
+}

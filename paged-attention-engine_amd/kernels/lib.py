@@ -79,6 +79,7 @@ def _declare(lib) -> None:
         "pae_hyper_collapse": [P, P, I, I, I, P],
         "pae_conv_norm_store": [I, P, L, P, L, I, I, P, P, P, P, P, P, L, I, I, I, I, I, I, F, P, I, I, P, P, P],
         "pae_latent_prepare": [I, P, L, P, L, I, I, I, I, I, I, I, P, I, F, P, P, P, P, I, I, P, P, P],
+        "pae_heads_product_few": [P, L, L, P, L, L, P, I, I, I, I, P],
         "pae_latent_attn_supported": [I, I, I],
         "pae_latent_attn_columns": [I, I],
         "pae_latent_attn_bf16": [P, L, P, L, P, P, P, I, I, P, P, I, I, I, I, I, F, I, I, P, P, P],
@@ -925,10 +926,26 @@ def gemm_plain_heads(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor) -> Non
                                             w.stride(0), None, 0, M, N, K, B, _stream()))
 
 
+HEADS_FEW_MAX_ROWS = 16
+
+
 def heads_product(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor) -> None:
     """out[:, h, :] = a[:, h, :] @ w[h]^T for every head h (shapes as for `gemm_plain_heads`).  bfloat16 with
     more rows than the few-row kernels take goes to the platform's batched matrix product, as the plain
-    products of that many rows do; everything else to this engine's own kernel."""
+    products of that many rows do; bfloat16 with up to 16 rows to a kernel that streams the weights once;
+    everything else to the plain product's batched entry."""
+    if a.dtype == torch.bfloat16 and 0 < a.shape[0] <= HEADS_FEW_MAX_ROWS:
+        # a few rows: one wavefront per (head, output feature), the weights read once (every wavefront reads all rows
+        # of its head: at 64 rows that costs more than the plain kernel's tiles, measured)
+        _not_while_recording("heads_product")
+        _gpu(out, a, w)
+        M, B, K_ = a.shape
+        N = w.shape[1]
+        assert w.shape == (B, N, K_) and w.is_contiguous() and w.dtype == a.dtype == out.dtype
+        assert out.shape == (M, B, N) and a.stride(2) == 1 and out.stride(2) == 1
+        _check(library().pae_heads_product_few(out.data_ptr(), out.stride(0), out.stride(1), a.data_ptr(), a.stride(0),
+                                               a.stride(1), w.data_ptr(), M, N, K_, B, _stream()))
+        return
     if a.dtype == torch.bfloat16 and a.shape[0] > SKINNY_MAX_ROWS and _RECORDING is None:
         # [B, M, K] x [B, K, N] on strided views: no copy of the operands; the result is copied into the view
         out.copy_(torch.bmm(a.transpose(0, 1), w.transpose(1, 2)).transpose(0, 1))
