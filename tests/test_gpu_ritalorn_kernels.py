@@ -264,7 +264,9 @@ def test_the_spelled_out_attention_and_the_one_by_matrices_agree():
 @pytest.mark.parametrize("H,D,R,V,C,dims,bs,T,size", [(3, 16, 8, 24, 40, 8, 16, 150, 20), (2, 24, 16, 8, 16, 8, 8, 100, 7),
                                                       (4, 32, 32, 32, 64, 32, 16, 330, 100), (1, 40, 24, 72, 72, 24, 16, 80, 0),
                                                       (2, 8, 4, 12, 300, 4, 16, 70, 33), (5, 32, 64, 32, 512, 64, 16, 200, 60),
-                                                      (20, 16, 32, 16, 64, 32, 32, 90, 0), (12, 16, 32, 16, 128, 32, 16, 75, 17)])
+                                                      (20, 16, 32, 16, 64, 32, 32, 90, 0), (12, 16, 32, 16, 128, 32, 16, 75, 17),
+                                                      (3, 16, 32, 16, 96, 32, 16, 300, 130), (2, 24, 64, 8, 192, 64, 16, 280, 0),
+                                                      (1, 16, 32, 16, 64, 32, 16, 100, 50)])
 @pytest.mark.parametrize("new", ["prompt", "portion", "single"])
 def test_latent_attention_from_projected_rows_to_heads(dtype, H, D, R, V, C, dims, bs, T, size, new):
     """Projected rows through the latent norm, the rotation, the page write, the fold of the queries, the attention over
