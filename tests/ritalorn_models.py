@@ -54,7 +54,7 @@ A = {"architecture": "Ritalorn", "vocab": 301, "width": 64, "norm": {"eps": 2e-6
 B = {"architecture": "Ritalorn", "vocab": 211, "width": 100, "norm": {"eps": 1e-5}, "streams": 1, "logit_softcap": None,
      "layers": [
          layer(attention(3, 3, 48, 80, 0.2, conv=1, mask=16), ff=130),
-         layer(latent(4, 20, 12, 36, 28, 0.25, base=250000.0, mask=640), ff=60),
+         layer(latent(4, 20, 12, 36, 28, 0.25, base=40000.0, mask=640), ff=60),
          layer(attention(3, 3, 48, 80, 0.3, conv=3, mask=40, kv_from=0), ff=70),
      ]}
 # C: heads of 64 and 32 with values as wide (shapes matrix-core kernels may take), two readers of one layer,
@@ -62,7 +62,7 @@ B = {"architecture": "Ritalorn", "vocab": 211, "width": 100, "norm": {"eps": 1e-
 C = {"architecture": "Ritalorn", "vocab": 400, "width": 128, "norm": {"eps": 1e-5}, "streams": 2, "logit_softcap": 30.0,
      "layers": [
          layer(attention(8, 2, 64, 64, 0.15, conv=3, mask=48), ff=192),
-         layer(latent(4, 32, 32, 32, 64, 0.15, base=3000.0, mask=40)),
+         layer(latent(5, 32, 32, 48, 128, 0.15, base=3000.0, mask=36)),
          layer(attention(8, 2, 64, 64, 0.2, conv=3, mask=1000, kv_from=0), ff=64),
          layer(attention(4, 4, 32, 32, 0.3, conv=2), ff=64),
          layer(attention(8, 2, 64, 64, 0.1, conv=4, mask=24, kv_from=0)),
