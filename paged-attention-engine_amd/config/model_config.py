@@ -128,7 +128,7 @@ class LatentMixerSpec(PartSpec):
     Per token the mixer's input is projected down to `kv_rank` + `rope_dim` features: the first
     kv_rank, RMS-normed with a weight, are the latent c; the rest are one rotated key part shared by all
     heads.  Head h's key is [W_uk_h c | rotated part], its value W_uv_h c; a query head has `nope_dim`
-    features that meet W_uk_h c and `rope_dim` rotated ones.  Only c and the rotated part are cached."""
+    features that meet W_uk_h c and `rope_dim` rotated ones.  The cache holds c and the rotated part, nothing per head."""
 
     hidden_size: int = 0
     num_heads: int = 0

@@ -20,7 +20,7 @@
 // as exp(sink) without a key or a value of its own (sinks null: none).
 //
 // And four more, for designs that have them: a mask in chunks (`chunked`: the `window` is then a
-// chunk length, and position p sees the keys from p - p % window on, chunks counted from position 0
+// chunk length, and position p sees the keys from p - p % window on, chunk borders at multiples of the length from the first token
 // of the sequence); a bias by distance, score -= slopes[head] * (p - key) (slopes null: none); a gate
 // on the output, out *= sigmoid(gate[token][head][feature]) (gate null: none); and values that are
 // the first `vd` features of the key rows themselves (`shared_kv`, one latent row per token that

@@ -20,7 +20,7 @@ with y the sublayer's output times a per-feature scale (`ls1`, `ls2`) and u = su
 the model's output norm on the sum of the copies; in "attention": biases on q, k, v and o, a causal
 convolution over time on q, k and v right after the projection, q and k divided by their root mean
 square per head without a weight, no rotation but score -= 2^(-8 (h + 1) / H) (i - j), a mask in chunks
-counted from position 0, a gate sigmoid(W_g x) on the heads before W_o; in "latent_attention": the latent
+whose borders are multiples of the chunk length in the token's own sequence, a gate sigmoid(W_g x) on the heads before W_o; in "latent_attention": the latent
 RMS-normed with a weight, the rotated parts turned in pairs (2i, 2i + 1) by p * base^(-2i / dims), a
 sliding window that includes the token itself; the feed-forward W_down(gelu_tanh(W_gate x) * W_up x);
 a head of its own.  A mixer without "mask" sees every earlier token.

@@ -29,7 +29,7 @@ And for designs that have them (`MixerSpec.convolved`, the path `_forward_convol
 convolution over time on every channel of q, k and v right after the projection, whose last
 taps - 1 inputs are per-request state next to the pages; every query and key head divided by its own
 root mean square (`qk_norm = "head"`, no weight); a bias by distance instead of a rotation,
-score -= 2^(-b (h + 1) / H) * (i - j); a mask in chunks counted from position 0 of the sequence
+score -= 2^(-b (h + 1) / H) * (i - j); a mask in chunks whose borders are multiples of the chunk length in the sequence
 (`mask = "chunk"`); a gate sigmoid(W_g x) on the concatenated heads before W_o, whose projection is
 part of the one product and which the attention kernel applies as it writes; and layers without
 key/value tensors that read an earlier layer's pages (`own_kv = False`).  Pages of such a layer are

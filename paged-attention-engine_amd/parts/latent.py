@@ -10,7 +10,7 @@ value W_uv_j c; query and shared key part are rotated by position; the score is
 over the keys the mask lets through (a sliding window, chunks, or every earlier key), an ordinary
 softmax, and W_o on the concatenated heads.
 
-Only c and the rotated part are cached, one row of kv_rank + rope_dim per token whatever the number
+What the cache holds of a token is c and the rotated part, one row of kv_rank + rope_dim whatever the number
 of heads (`paged_spec`: one tensor "latent" [PAGE][kv_rank + rope_dim]).  The heads' keys and values
 are never formed: since q_nope . (W_uk_j c) = (W_uk_j^T q_nope) . c, the query is folded into latent
 space once per token ([W_uk_j^T q_nope | q_rot], kv_rank + rope_dim wide), the attention kernel scores
