@@ -123,11 +123,15 @@ __global__ __launch_bounds__(256, 1) void latent_attn_kernel(
         pb[i] = bf16_bits(p);
       }
       l[ct] = l[ct] * alpha + psum;
+      // the output tile is rescaled only if some column's maximum rose (a product with 1 changes nothing, so the
+      // result is the same bit for bit; after the first tiles most tiles raise no maximum)
+      if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
 #pragma unroll
-      for (int t = 0; t < VS / 16; ++t) {
-        acc[ct][t] *= alpha;
-        acc[ct][t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf[t], pb, acc[ct][t], 0, 0, 0);
+        for (int t = 0; t < VS / 16; ++t) acc[ct][t] *= alpha;
       }
+#pragma unroll
+      for (int t = 0; t < VS / 16; ++t)
+        acc[ct][t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf[t], pb, acc[ct][t], 0, 0, 0);
     }
   };
   int key0 = lo + 16 * wave;  // the same in every lane of a wavefront: the branches on it are uniform
